@@ -48,12 +48,68 @@ class KVCheckpoint:
     data: torch.Tensor  # pinned host [n_layers, n_pages, page_shorts] bf16
 
 
+class GQALayout:
+    """Per layer a K pool [P, n_kv, D/8, PS, 8] and a V pool [P, n_kv, PS, D]
+    (the layouts the GQA attention kernels stream)."""
+
+    def __init__(self, n_layers: int, n_kv: int, head_dim: int):
+        assert head_dim % 8 == 0
+        self.n_layers, self.n_kv, self.head_dim = n_layers, n_kv, head_dim
+
+    def alloc(self, n_pages, page_size, device, dtype):
+        return [(torch.zeros(n_pages, self.n_kv, self.head_dim // 8,
+                             page_size, 8, dtype=dtype, device=device),
+                 torch.zeros(n_pages, self.n_kv, page_size, self.head_dim,
+                             dtype=dtype, device=device))
+                for _ in range(self.n_layers)]
+
+    def page_elems(self, page_size: int) -> int:
+        return 2 * self.n_kv * self.head_dim * page_size
+
+    def gather(self, entry, staging, page_ids):
+        ops.gather_kv_pages(staging, entry[0], entry[1], page_ids)
+
+    def scatter(self, entry, staging, page_ids):
+        ops.scatter_kv_pages(entry[0], entry[1], staging, page_ids)
+
+
+class LatentLayout:
+    """Per layer ONE pool [P, PS, R_l] of cached attention latents (row =
+    token); R_l may differ between layers. Checkpoint images are sized by
+    the widest layer."""
+
+    def __init__(self, ranks: List[int]):
+        self.ranks = list(ranks)
+        self.n_layers = len(self.ranks)
+
+    def alloc(self, n_pages, page_size, device, dtype):
+        return [(torch.zeros(n_pages, page_size, r, dtype=dtype,
+                             device=device),) for r in self.ranks]
+
+    def page_elems(self, page_size: int) -> int:
+        return max(self.ranks) * page_size
+
+    def gather(self, entry, staging, page_ids):
+        pool = entry[0]
+        n = pool.size(1) * pool.size(2)
+        staging[:, :n] = pool.index_select(0, page_ids.long()).view(-1, n)
+
+    def scatter(self, entry, staging, page_ids):
+        pool = entry[0]
+        n = pool.size(1) * pool.size(2)
+        pool.index_copy_(0, page_ids.long(),
+                         staging[:, :n].reshape(-1, pool.size(1),
+                                                pool.size(2)))
+
+
 class KVCacheManager:
     def __init__(self, n_layers: int, n_kv: int, head_dim: int, page_size: int,
                  n_pages: int, device="cpu", dtype=torch.bfloat16,
                  max_slots: int = 1024, max_pages_per_seq: int = 512,
-                 mirrors: Optional[bool] = None):
-        assert head_dim % 8 == 0
+                 mirrors: Optional[bool] = None, layout=None):
+        # layout: what one layer caches per page (default: GQA K/V planes)
+        self.layout = layout or GQALayout(n_layers, n_kv, head_dim)
+        n_layers = self.layout.n_layers
         self.n_layers = n_layers
         self.n_kv = n_kv
         self.head_dim = head_dim
@@ -64,13 +120,10 @@ class KVCacheManager:
         # token (2x the agents per GPU) with OCP e4m3 storage, vLLM-style
         # scale-free semantics (e4m3 range +-448 covers post-norm K/V)
         self.dtype = dtype
-        self.k_caches: List[torch.Tensor] = []
-        self.v_caches: List[torch.Tensor] = []
-        for _ in range(n_layers):
-            self.k_caches.append(torch.zeros(
-                n_pages, n_kv, head_dim // 8, page_size, 8, dtype=dtype, device=device))
-            self.v_caches.append(torch.zeros(
-                n_pages, n_kv, page_size, head_dim, dtype=dtype, device=device))
+        self.caches = self.layout.alloc(n_pages, page_size, device, dtype)
+        if isinstance(self.layout, GQALayout):
+            self.k_caches: List[torch.Tensor] = [c[0] for c in self.caches]
+            self.v_caches: List[torch.Tensor] = [c[1] for c in self.caches]
         # page 0 is reserved as the scratch page: hipGraph-padded decode rows
         # write their garbage K/V there (see llm.ModelInstance._device_decode)
         self._free: List[int] = list(range(n_pages - 1, 0, -1))
@@ -84,7 +137,7 @@ class KVCacheManager:
         self._refs: Dict[int, int] = {}
         self._lock = threading.RLock()
         # shorts per page per layer: K plane + V plane
-        self.page_shorts = 2 * n_kv * head_dim * page_size
+        self.page_shorts = self.layout.page_elems(page_size)
         # ---- device mirrors for the in-graph decode step ----
         # dev_page_table[slot] / dev_seq_lens[slot] are the ground truth the
         # captured decode graph reads; host bookkeeping mirrors them. On GPU
@@ -122,7 +175,7 @@ class KVCacheManager:
         return self.n_pages - self.free_pages
 
     def kv_caches(self) -> List[Tuple[torch.Tensor, torch.Tensor]]:
-        return list(zip(self.k_caches, self.v_caches))
+        return list(self.caches)
 
     def has_seq(self, seq_id: str) -> bool:
         with self._lock:
@@ -139,7 +192,7 @@ class KVCacheManager:
             if not s:
                 return 0
             return (len(s.pages) * self.page_shorts * self.n_layers *
-                    self.k_caches[0].element_size())
+                    self.caches[0][0].element_size())
 
     # ---------- allocation ----------
 
@@ -416,15 +469,13 @@ class KVCacheManager:
             staging = torch.empty(n, self.page_shorts, dtype=self.dtype,
                                   device=self.device)
             for li in range(self.n_layers):
-                ops.gather_kv_pages(staging, self.k_caches[li], self.v_caches[li],
-                                    page_ids)
+                self.layout.gather(self.caches[li], staging, page_ids)
                 host[li].copy_(staging, non_blocking=True)
             torch.cuda.synchronize()
         else:
             staging = torch.empty(n, self.page_shorts, dtype=self.dtype)
             for li in range(self.n_layers):
-                ops.gather_kv_pages(staging, self.k_caches[li], self.v_caches[li],
-                                    page_ids)
+                self.layout.gather(self.caches[li], staging, page_ids)
                 host[li].copy_(staging)
         if free:
             self.free_seq(seq_id)
@@ -447,8 +498,7 @@ class KVCacheManager:
         is_gpu = str(self.device) not in ("cpu",)
         for li in range(self.n_layers):
             staging = ckpt.data[li].to(self.device, non_blocking=is_gpu)
-            ops.scatter_kv_pages(self.k_caches[li], self.v_caches[li],
-                                 staging, page_ids)
+            self.layout.scatter(self.caches[li], staging, page_ids)
         self.push_dev(seq_id)
         if is_gpu:
             torch.cuda.synchronize()

@@ -138,8 +138,23 @@ class ModelInstance:
             assert par.is_tp() and par.tp_size() == self.tp_size, (
                 f"tp_degree={self.tp_size} requires torchrun world of that size")
         model_cls = model_cls or LlamaForCausalLM
-        self.model = model_cls(cfg, device=device,
-                               tp_rank=self.tp_rank, tp_size=self.tp_size)
+        # compute dtype: bf16 serving default; float32 only for model
+        # families whose kernels are typed for it
+        dt_s = str(engine_cfg.get("dtype", "bf16") or "bf16")
+        if dt_s in ("bf16", "bfloat16"):
+            self.dtype = torch.bfloat16
+        elif dt_s in ("fp32", "float32"):
+            self.dtype = torch.float32
+        else:
+            raise ValueError(f"unsupported engine dtype {dt_s!r}")
+        import inspect
+        mk = {}
+        if "dtype" in inspect.signature(model_cls.__init__).parameters:
+            mk["dtype"] = self.dtype
+        elif self.dtype != torch.bfloat16:
+            raise ValueError(f"{model_cls.__name__} runs in bf16 only")
+        self.model = model_cls(cfg, device=device, tp_rank=self.tp_rank,
+                               tp_size=self.tp_size, **mk)
         if self.tp_size > 1:
             self.model.tp_group = par.tp_group()
         if weights_path:
@@ -161,7 +176,6 @@ class ModelInstance:
                       else 0.5 if (fp8 or dq == "fp8") else 1.0)
             free, total = torch.cuda.mem_get_info()
             if param_bytes * (1.0 + factor) < 0.75 * total:
-                import inspect
                 sig = inspect.signature(self.model.pack_decode_weights)
                 if "expert_fp8" in sig.parameters:
                     self.model.pack_decode_weights(expert_fp8=fp8,
@@ -178,17 +192,25 @@ class ModelInstance:
             kv_dtype = torch.bfloat16
         else:
             raise ValueError(f"unsupported kv_dtype {kv_dtype_s!r}")
+        if self.dtype == torch.float32:
+            kv_dtype = torch.float32
         n_pages = self._pool_pages(cfg, page_size, device, engine_cfg,
                                    self.tp_size)
         # sequence-slot budget: device page-table/length mirrors are tiny
         # (2048 slots x 512 pages x 4 B = 4 MB), so default well above the
         # largest measured concurrency (1k+ agents per GPU with fp8 KV)
         max_seqs = int(engine_cfg.get("max_seqs", 2048))
+        # what a layer caches per token is the model family's business:
+        # GQA K/V planes by default, or the layout the config names
+        layout = cfg.cache_layout() if hasattr(cfg, "cache_layout") else None
         self.kvm = KVCacheManager(cfg.n_layers,
-                                  max(cfg.n_kv_heads // self.tp_size, 1),
-                                  cfg.head_dim, page_size, n_pages,
-                                  device=device, dtype=kv_dtype,
-                                  max_slots=max_seqs,
+                                  max(getattr(cfg, "n_kv_heads", 1)
+                                      // self.tp_size, 1),
+                                  getattr(cfg, "head_dim", 8), page_size,
+                                  n_pages, device=device, dtype=kv_dtype,
+                                  max_slots=max_seqs, layout=layout,
+                                  max_pages_per_seq=int(engine_cfg.get(
+                                      "max_pages_per_seq", 512)),
                                   mirrors=(device.startswith("cuda") or bool(
                                       engine_cfg.get("async_decode_emulate",
                                                      False))))
@@ -296,7 +318,14 @@ class ModelInstance:
     @staticmethod
     def _pool_pages(cfg: LlamaConfig, page_size: int, device: str,
                     engine_cfg: Dict[str, Any], tp_size: int = 1) -> int:
+        # explicit token budget: exactly that many tokens' worth of pages
+        # plus the reserved scratch page 0
+        pool_tokens = int(engine_cfg.get("kv_pool_tokens", 0) or 0)
+        if pool_tokens > 0:
+            return -(-pool_tokens // page_size) + 1
         eb = 1 if str(engine_cfg.get("kv_dtype", "bf16")).startswith(("fp8", "e4m3")) else 2
+        if str(engine_cfg.get("dtype", "bf16")) in ("fp32", "float32"):
+            eb = 4
         bytes_per_page = cfg.kv_bytes_per_token(eb) * page_size // max(tp_size, 1)
         pool_gb = float(engine_cfg.get("kv_pool_gb", 0.0))
         if device.startswith("cuda") and pool_gb <= 0:
@@ -862,8 +891,11 @@ class ModelInstance:
             b <<= 1
         return b
 
-    def _prefill_exec(self, plan) -> torch.Tensor:
-        """Runs identically on every TP rank (plan = seq ids + tokens)."""
+    def _prefill_exec(self, plan, want=None) -> torch.Tensor:
+        """Runs identically on every TP rank (plan = seq ids + tokens).
+        Returns one logits row per plan row (its last token), or, when
+        `want` lists per-row token offsets, one row per wanted offset in
+        plan order."""
         dev = self.device
         ids: List[int] = []
         positions: List[int] = []
@@ -931,9 +963,13 @@ class ModelInstance:
             max_qlen=max(q_lens),
         )
         input_ids = torch.tensor(ids, dtype=torch.long, device=dev)
-        last_rows = torch.tensor(
-            [s + l - 1 for s, l in zip(q_starts[:n_real], q_lens[:n_real])],
-            dtype=torch.long, device=dev)
+        if want is None:
+            rows_l = [s + l - 1
+                      for s, l in zip(q_starts[:n_real], q_lens[:n_real])]
+        else:
+            rows_l = [q_starts[i] + int(o) for i in range(n_real)
+                      for o in want[i]]
+        last_rows = torch.tensor(rows_l, dtype=torch.long, device=dev)
         c0 = time.thread_time()
         out = self.model(input_ids, md, self.kvm.kv_caches(), last_rows)
         fwd_cpu = (time.thread_time() - c0) * 1000.0
@@ -943,6 +979,37 @@ class ModelInstance:
         if mn is None or fwd_cpu < mn:
             self._phase_ms["pf_fwd_cpu_min_ms"] = fwd_cpu
         return out
+
+    def forward_step(self, entries, want) -> torch.Tensor:
+        """Teacher-forced engine step: entries = [(seq_id, tokens)] are the
+        next tokens of live sequences (sequences are created on first
+        use), all run as ONE batch on top of the cache earlier steps left;
+        want[i] lists the offsets into entries[i]'s tokens whose logits
+        are returned ([n_wanted, vocab], entry order). A step made only of
+        single tokens of sequences that already hold context is a decode
+        step and takes the decode path (device-side append + captured
+        graph on GPU); anything else — prompt portions, alone or beside
+        single tokens — takes the varlen path. Nothing is sampled."""
+        if self._spec is not None or self._pf_pending is not None:
+            self.drain_async()
+        for seq_id, _toks in entries:
+            if not self.kvm.has_seq(seq_id):
+                self._bind_seq(seq_id, None)
+        decode = all(len(t) == 1 and self.kvm.seq_len(s) > 0
+                     for s, t in entries)
+        if decode and len(entries) <= max(self.max_decode_batch, 1):
+            logits = self._decode_exec([(s, t[0]) for s, t in entries])
+            keep = [i for i, w in enumerate(want) if len(w) > 0]
+            if len(keep) < len(entries):
+                logits = logits[keep]
+            return logits
+        plan = [(s, list(t), False, None) for s, t in entries]
+        return self._prefill_exec(plan, want=[list(w) for w in want])
+
+    def release(self, seq_id: str) -> None:
+        """Give a finished sequence's pages and slot back to the pool."""
+        if self.kvm.has_seq(seq_id):
+            self.kvm.free_seq(seq_id)
 
     # ---------- device-side decode (hipGraph) ----------
 
@@ -1311,17 +1378,16 @@ class LLMEngine:
         self._lock = threading.RLock()
         self.tp_size = int(self.engine_cfg.get("tp_degree", 1))
         self.tp_rank = par.tp_rank() if self.tp_size > 1 else 0
-        if device == "cuda" and torch.cuda.is_available():
-            if not ops.hip_available():
-                raise RuntimeError(
-                    "GPU engine requires the gfx950 HIP extension "
-                    "(python -m agentainer_amd.ops.build)")
+        # each model family checks for the HIP extension ITS kernels live
+        # in when an instance is made (_make_instance)
 
     # ---------- model registry ----------
 
     def validate_model(self, model: str) -> None:
         from ..models.mixtral import MIXTRAL_CONFIGS
-        if model in LLAMA_CONFIGS or model in MIXTRAL_CONFIGS:
+        from ..models.lelitar import LELITAR_CONFIGS
+        if (model in LLAMA_CONFIGS or model in MIXTRAL_CONFIGS
+                or model in LELITAR_CONFIGS):
             return
         from .echo import ECHO_MODELS
         if model in ECHO_MODELS:
@@ -1331,10 +1397,25 @@ class LLMEngine:
         from ..models.mixtral import MIXTRAL_CONFIGS as _MC
         raise ModelNotFound(
             f"unknown model {model!r}; known: "
-            f"{sorted(LLAMA_CONFIGS) + sorted(_MC)} + echo")
+            f"{sorted(LLAMA_CONFIGS) + sorted(_MC) + sorted(LELITAR_CONFIGS)}"
+            " + echo")
 
     def _make_instance(self, model: str) -> ModelInstance:
         from ..models.mixtral import MIXTRAL_CONFIGS, make_mixtral_instance
+        from ..models.lelitar import (LELITAR_CONFIGS, is_lelitar_checkpoint,
+                                      make_lelitar_instance)
+        if model in LELITAR_CONFIGS:
+            return make_lelitar_instance(model, self.device, self.engine_cfg)
+        if os.path.isdir(os.path.expanduser(model)) and is_lelitar_checkpoint(
+                os.path.expanduser(model)):
+            # the checkpoint's config.json names its architecture
+            return make_lelitar_instance(model, self.device, self.engine_cfg,
+                                         weights_path=os.path.expanduser(model))
+        if (self.device.startswith("cuda") and torch.cuda.is_available()
+                and not ops.hip_available()):
+            raise RuntimeError(
+                "GPU engine requires the gfx950 HIP extension "
+                "(python -m agentainer_amd.ops.build)")
         if model in LLAMA_CONFIGS:
             return ModelInstance(model, LLAMA_CONFIGS[model], self.device,
                                  self.engine_cfg)

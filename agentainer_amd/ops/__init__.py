@@ -228,7 +228,9 @@ def linear(x: torch.Tensor, w: torch.Tensor,
     N = w.size(0)
     tuned = _SKINNY_SHAPES.get((N, K))
     if (x.is_cuda and M <= 64 and N % 64 == 0 and K % 256 == 0
-            and (tuned is not None or SKINNY_FORCED) and not SKINNY_DISABLED):
+            and x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16
+            and (tuned is not None or SKINNY_FORCED) and not SKINNY_DISABLED
+            and hip_available()):
         mod = _dispatch("skinny_gemm", x)
         split, kc = tuned if tuned else (_skinny_split(N // 64, K), 128)
         if SKINNY_KC:
@@ -383,3 +385,137 @@ def scatter_kv_pages(k_cache, v_cache, src, page_ids):
         mod.scatter_kv_pages(k_cache, v_cache, src, page_ids)
     else:
         reference.scatter_kv_pages(k_cache, v_cache, src, page_ids)
+
+
+# ---------------------------------------------------------------------
+# Grouped norm / latent window attention / sigmoid-routed experts.
+# These kernels live in their own extension (_hip_latent.so) so a model
+# that needs only them compiles only them. Same policy as above: on a GPU
+# the extension is required, on CPU the fp32 references run.
+# ---------------------------------------------------------------------
+
+_latent = None
+_latent_err: Optional[str] = None
+
+
+def _load_latent():
+    global _latent, _latent_err
+    if _latent is not None or _latent_err is not None:
+        return _latent
+    so = os.path.join(os.path.dirname(__file__), "_hip_latent.so")
+    if not os.path.exists(so):
+        _latent_err = (f"HIP extension not built ({so} missing); run "
+                       "python -m agentainer_amd.ops.build latent")
+        return None
+    try:
+        import importlib.util
+
+        spec = importlib.util.spec_from_file_location(
+            "agentainer_amd.ops._hip_latent", so)
+        mod = importlib.util.module_from_spec(spec)
+        spec.loader.exec_module(mod)
+        _latent = mod
+    except Exception as exc:  # noqa: BLE001
+        _latent_err = f"HIP extension failed to load: {exc}"
+    return _latent
+
+
+def latent_available() -> bool:
+    return _load_latent() is not None
+
+
+def _dispatch_latent(name: str, t: torch.Tensor):
+    if t.is_cuda:
+        mod = _load_latent()
+        if mod is None:
+            raise RuntimeError(
+                f"op {name!r} on GPU requires the gfx950 HIP extension: "
+                f"{_latent_err}")
+        return mod
+    return None
+
+
+def residual_grouped_rmsnorm(x_res, add_a, add_b, mult: float, weights, outs,
+                             groups: int, eps: float):
+    """fp32 residual update fused with up to two grouped RMS norms of the
+    updated stream (see reference.residual_grouped_rmsnorm)."""
+    mod = _dispatch_latent("residual_grouped_rmsnorm", x_res)
+    if mod:
+        mod.residual_grouped_rmsnorm(
+            x_res, add_a, add_b, float(mult), weights[0], outs[0],
+            weights[1] if len(weights) > 1 else None,
+            outs[1] if len(outs) > 1 else None, int(groups), float(eps))
+    else:
+        reference.residual_grouped_rmsnorm(x_res, add_a, add_b, mult, weights,
+                                           outs, groups, eps)
+    return outs
+
+
+def latent_norm_append(proj, q_off, q_rank, kv_off, kv_rank, wq, wkv, eps,
+                       cq_out, cache, slot_mapping):
+    mod = _dispatch_latent("latent_norm_append", proj)
+    if mod:
+        mod.latent_norm_append(proj, int(q_off), int(q_rank), int(kv_off),
+                               int(kv_rank), wq, wkv, float(eps), cq_out,
+                               cache, slot_mapping)
+    else:
+        reference.latent_norm_append(proj, q_off, q_rank, kv_off, kv_rank, wq,
+                                     wkv, eps, cq_out, cache, slot_mapping)
+
+
+# AGENTAINER_LATENT_SIMPLE=1 forces the one-wave-per-row kernel (A/B and
+# numerics cross-checks against the MFMA tile kernel)
+LATENT_SIMPLE = os.environ.get("AGENTAINER_LATENT_SIMPLE", "0") == "1"
+
+
+def latent_window_attention(out, q_lat, cache, page_table, seq_lens,
+                            query_starts, query_lens, scale: float,
+                            window: int, max_qlen: int = 1):
+    mod = _dispatch_latent("latent_window_attention", q_lat)
+    if mod:
+        mod.latent_window_attention(out, q_lat, cache, page_table, seq_lens,
+                                    query_starts, query_lens, float(scale),
+                                    int(window), int(max_qlen),
+                                    bool(LATENT_SIMPLE))
+    else:
+        reference.latent_window_attention(out, q_lat, cache, page_table,
+                                          seq_lens, query_starts, query_lens,
+                                          scale, window)
+    return out
+
+
+def sigmoid_gate_mul(out, a, g):
+    mod = _dispatch_latent("sigmoid_gate_mul", a)
+    if mod:
+        mod.sigmoid_gate_mul(out, a, g)
+    else:
+        reference.sigmoid_gate_mul(out, a, g)
+    return out
+
+
+def act_mul(out, gate, up, act: str):
+    """out = act(gate) * up with act in {"relu", "silu"}; bf16 or fp32."""
+    mod = _dispatch_latent("act_mul", gate)
+    if mod:
+        mod.act_mul(out, gate, up, {"relu": 0, "silu": 1}[act])
+    else:
+        reference.act_mul(out, gate, up, act)
+    return out
+
+
+def sigmoid_topk_route(weight, logits, top: int):
+    mod = _dispatch_latent("sigmoid_topk_route", logits)
+    if mod:
+        mod.sigmoid_topk_route(weight, logits, int(top))
+    else:
+        reference.sigmoid_topk_route(weight, logits, top)
+    return weight
+
+
+def routed_scaled_silu_mul(out, gu, weight):
+    mod = _dispatch_latent("routed_scaled_silu_mul", gu)
+    if mod:
+        mod.routed_scaled_silu_mul(out, gu, weight)
+    else:
+        reference.routed_scaled_silu_mul(out, gu, weight)
+    return out

@@ -31,6 +31,15 @@ OUT = os.path.join(HERE, "_hip_ops_asan.so" if ASAN else "_hip_ops.so")
 OBJ_DIR = os.path.join(HERE, "_build_asan" if ASAN else "_build")
 ARCH = os.environ.get("PYTORCH_ROCM_ARCH", "gfx950")
 
+# the latent-attention family's kernels build into their own module so a
+# deployment that serves only that family compiles only these
+LATENT_SOURCES = [
+    "latent_bindings.cpp",
+    "grouped_norm.hip",
+    "latent_attn.hip",
+    "routed_ffn.hip",
+]
+
 SOURCES = [
     "bindings.cpp",
     "rmsnorm.hip",
@@ -48,7 +57,20 @@ def _newest(paths):
     return max(os.path.getmtime(p) for p in paths if os.path.exists(p))
 
 
-def needs_build() -> bool:
+def _target(target: str):
+    """(output .so, object dir, sources, module name) of a build target."""
+    if target == "latent":
+        sfx = "_asan" if ASAN else ""
+        return (os.path.join(HERE, f"_hip_latent{sfx}.so"),
+                os.path.join(HERE, "_build_latent" + sfx), LATENT_SOURCES,
+                "_hip_latent")
+    if target != "core":
+        raise ValueError(f"unknown build target {target!r}")
+    return OUT, OBJ_DIR, SOURCES, "_hip_ops"
+
+
+def needs_build(target: str = "core") -> bool:
+    OUT, _obj, SOURCES, _name = _target(target)
     if not os.path.exists(OUT):
         return True
     srcs = [os.path.join(CSRC, s) for s in SOURCES]
@@ -57,8 +79,13 @@ def needs_build() -> bool:
     return _newest(srcs) > os.path.getmtime(OUT)
 
 
-def build(verbose: bool = True, force: bool = False) -> str:
-    if not force and not needs_build():
+def build(verbose: bool = True, force: bool = False,
+          target: str = "core") -> str:
+    if target == "all":
+        build(verbose, force, "core")
+        return build(verbose, force, "latent")
+    OUT, OBJ_DIR, SOURCES, modname = _target(target)
+    if not force and not needs_build(target):
         return OUT
     os.makedirs(OBJ_DIR, exist_ok=True)
     torch_inc = cpp_extension.include_paths()
@@ -68,7 +95,9 @@ def build(verbose: bool = True, force: bool = False) -> str:
     cxx_flags = [
         "-O3", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}",
         "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1",
-        "-DTORCH_EXTENSION_NAME=_hip_ops",
+        f"-DTORCH_EXTENSION_NAME={modname}",
+        # packed-fp32 VALU forms are kept out of generated code
+        "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
         "-D_GLIBCXX_USE_CXX11_ABI=1",
         "-fno-gpu-rdc",
         "-Wno-unused-result",
@@ -105,12 +134,16 @@ def build(verbose: bool = True, force: bool = False) -> str:
                "-ltorch_hip", "-lc10_hip", f"-Wl,-rpath,{torch_lib}"])
     if verbose:
         print("[ops.build]", " ".join(link), flush=True)
+    tmp_out = OUT + f".tmp{os.getpid()}"
+    link[link.index(OUT)] = tmp_out
     res = subprocess.run(link, capture_output=True)
     if res.returncode != 0:
         raise RuntimeError(f"link failed:\n{res.stdout.decode()}\n{res.stderr.decode()}")
+    os.replace(tmp_out, OUT)
     return OUT
 
 
 if __name__ == "__main__":
-    build(force="--force" in sys.argv)
-    print(f"built {OUT}")
+    targets = [a for a in sys.argv[1:] if not a.startswith("-")] or ["all"]
+    for t in targets:
+        print("built", build(force="--force" in sys.argv, target=t))

@@ -180,3 +180,134 @@ def scatter_kv_pages(k_cache: torch.Tensor, v_cache: torch.Tensor,
     for i, p in enumerate(page_ids.tolist()):
         k_cache[p] = flat[i * 2 * plane:(i * 2 + 1) * plane].view_as(k_cache[p])
         v_cache[p] = flat[(i * 2 + 1) * plane:(i + 1) * 2 * plane].view_as(v_cache[p])
+
+
+# ---------------------------------------------------------------------
+# Grouped norm, latent window attention, sigmoid-routed experts
+# (fp32 math; outputs take the dtype of the tensor they are written to)
+# ---------------------------------------------------------------------
+
+def residual_grouped_rmsnorm(x_res: torch.Tensor, add_a, add_b, mult: float,
+                             weights, outs, groups: int, eps: float) -> None:
+    """x_res (fp32, in place) += mult * (add_a + add_b); then for every
+    (w, out) pair: out = x_res / sqrt(mean_g(x_res^2) + eps) * w, the mean
+    taken separately over each of `groups` equal consecutive parts."""
+    if add_a is not None or add_b is not None:
+        s = torch.zeros_like(x_res)
+        if add_a is not None:
+            s = s + add_a.float()
+        if add_b is not None:
+            s = s + add_b.float()
+        x_res.add_(s * mult)
+    T, W = x_res.shape
+    parts = x_res.view(T, groups, W // groups)
+    unit = (parts * torch.rsqrt(parts.pow(2).mean(-1, keepdim=True) + eps)
+            ).reshape(T, W)
+    for w, out in zip(weights, outs):
+        out.copy_((unit * w.float()).to(out.dtype))
+
+
+def latent_norm_append(proj: torch.Tensor, q_off: int, q_rank: int,
+                       kv_off: int, kv_rank: int, wq: torch.Tensor,
+                       wkv: torch.Tensor, eps: float, cq_out: torch.Tensor,
+                       cache: torch.Tensor, slot_mapping: torch.Tensor) -> None:
+    """RMS-norm the query latent and the key/value latent held in two
+    column ranges of `proj`; the first goes to cq_out, the second into
+    the paged latent pool cache[P, PS, Rp] at each token's slot (columns
+    past kv_rank are zero-filled; slot < 0 skips the append)."""
+    def unit(v):
+        return v * torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + eps)
+
+    cq = proj[:, q_off:q_off + q_rank].float()
+    cq_out.copy_((unit(cq) * wq.float()).to(cq_out.dtype))
+    c = proj[:, kv_off:kv_off + kv_rank].float()
+    c = (unit(c) * wkv.float()).to(cache.dtype)
+    PS, Rp = cache.size(1), cache.size(2)
+    flat = cache.view(-1, Rp)
+    ok = slot_mapping >= 0
+    rows = slot_mapping[ok].long()
+    flat[rows, :kv_rank] = c[ok]
+    if Rp > kv_rank:
+        flat[rows, kv_rank:] = 0
+
+
+def latent_window_attention(out: torch.Tensor, q_lat: torch.Tensor,
+                            cache: torch.Tensor, page_table: torch.Tensor,
+                            seq_lens: torch.Tensor, query_starts,
+                            query_lens, scale: float, window: int) -> None:
+    """Multi-query attention in latent space: every head's query q_lat[h, t]
+    (already mapped into the latent basis) scores the cached latents
+    themselves, and the output is the softmax-weighted sum of the same
+    latents. A query at position p sees keys at p - window < j <= p.
+    q_lat/out: [H, T, Rp]; cache [P, PS, Rp]. query_starts/query_lens None
+    means one new token per sequence (decode)."""
+    H = q_lat.size(0)
+    PS, Rp = cache.size(1), cache.size(2)
+    flat = cache.view(-1, Rp)
+    B = seq_lens.numel()
+    for b in range(B):
+        total = int(seq_lens[b])
+        qlen = 1 if query_lens is None else int(query_lens[b])
+        start = b if query_starts is None else int(query_starts[b])
+        if total <= 0 or qlen == 0:
+            if total <= 0 and query_lens is None:
+                out[:, start] = 0
+            continue
+        ctx = total - qlen
+        lo = max(0, ctx - window + 1)
+        pos = torch.arange(lo, total)
+        rows = (page_table[b, (pos // PS).long()].long() * PS + pos % PS)
+        C = flat[rows].float()                          # [n, Rp]
+        Q = q_lat[:, start:start + qlen].float()        # [H, qlen, Rp]
+        s = torch.einsum("hqr,nr->hqn", Q, C) * scale
+        qpos = (ctx + torch.arange(qlen)).view(1, qlen, 1)
+        kpos = pos.view(1, 1, -1)
+        seen = (kpos <= qpos) & (qpos - kpos < window)
+        s = s.masked_fill(~seen, float("-inf"))
+        p = torch.softmax(s, dim=-1)
+        out[:, start:start + qlen] = torch.einsum("hqn,nr->hqr", p, C
+                                                  ).to(out.dtype)
+
+
+def sigmoid_gate_mul(out: torch.Tensor, a: torch.Tensor, g: torch.Tensor) -> None:
+    """out[t, h*E + e] = a[h, t, e] * sigmoid(g[t, h*E + e])."""
+    H, T, E = a.shape
+    av = a.permute(1, 0, 2).reshape(T, H * E).float()
+    out.copy_((av * torch.sigmoid(g.float())).to(out.dtype))
+
+
+def act_mul(out: torch.Tensor, gate: torch.Tensor, up: torch.Tensor,
+            act: str) -> None:
+    g = gate.float()
+    if act == "relu":
+        a = torch.relu(g)
+    elif act == "silu":
+        a = g * torch.sigmoid(g)
+    else:
+        raise ValueError(act)
+    out.copy_((a * up.float()).to(out.dtype))
+
+
+def sigmoid_topk_route(weight: torch.Tensor, logits: torch.Tensor,
+                       top: int) -> None:
+    """weight[t, e] = sigmoid(logits[t, e]) for the `top` largest entries
+    of row t (ties: lowest index first), 0 elsewhere. fp32 throughout."""
+    s = torch.sigmoid(logits.float())
+    val, idx = s.topk(top, dim=-1)
+    weight.zero_()
+    weight.scatter_(1, idx, val)
+
+
+def routed_scaled_silu_mul(out: torch.Tensor, gu: torch.Tensor,
+                           weight: torch.Tensor) -> None:
+    """Stacked-expert activation with the routing weight applied on the
+    INPUT side: gu [T, E, 2F] holds every expert's gate|up projections of
+    the unscaled input, so the scaled-input projections are w*gate and
+    w*up; out[t, e, :] = silu(w g) * (w u), which is 0 where w == 0."""
+    T, E = weight.shape
+    F_ = gu.size(-1) // (2 * E)
+    g3 = gu.view(T, E, 2 * F_).float()
+    w = weight.view(T, E, 1).float()
+    g = g3[..., :F_] * w
+    u = g3[..., F_:] * w
+    out.copy_((g * torch.sigmoid(g) * u).view(T, E * F_).to(out.dtype))
