@@ -1,0 +1,40 @@
+// pybind11 bindings: grouped norm, latent window attention, routed experts.
+#include <torch/extension.h>
+
+void residual_grouped_rmsnorm(torch::Tensor x, c10::optional<torch::Tensor> a,
+                              c10::optional<torch::Tensor> b, double mult,
+                              torch::Tensor w1, torch::Tensor o1,
+                              c10::optional<torch::Tensor> w2,
+                              c10::optional<torch::Tensor> o2, long groups,
+                              double eps);
+void latent_norm_append(torch::Tensor proj, long q_off, long q_rank,
+                        long kv_off, long kv_rank, torch::Tensor wq,
+                        torch::Tensor wkv, double eps, torch::Tensor cq_out,
+                        torch::Tensor cache, torch::Tensor slot_mapping);
+void latent_window_attention(torch::Tensor out, torch::Tensor q_lat,
+                             torch::Tensor cache, torch::Tensor page_table,
+                             torch::Tensor seq_lens,
+                             c10::optional<torch::Tensor> query_starts,
+                             c10::optional<torch::Tensor> query_lens,
+                             double scale, long window, long max_qlen,
+                             bool force_simple);
+void sigmoid_gate_mul(torch::Tensor out, torch::Tensor a, torch::Tensor g);
+void act_mul(torch::Tensor out, torch::Tensor gate, torch::Tensor up, long act);
+void sigmoid_topk_route(torch::Tensor weight, torch::Tensor logits, long top);
+void routed_scaled_silu_mul(torch::Tensor out, torch::Tensor gu,
+                            torch::Tensor weight);
+
+PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
+  m.doc() = "agentainer_amd CDNA4 (gfx950) latent-attention family kernels";
+  m.def("residual_grouped_rmsnorm", &residual_grouped_rmsnorm,
+        "x += mult*(a+b); grouped RMS norms of x (fp32 residual)");
+  m.def("latent_norm_append", &latent_norm_append,
+        "RMS-norm query/kv latents; append the kv latent to the paged pool");
+  m.def("latent_window_attention", &latent_window_attention,
+        "sliding-window multi-query attention over paged latents");
+  m.def("sigmoid_gate_mul", &sigmoid_gate_mul, "heads * sigmoid(gate)");
+  m.def("act_mul", &act_mul, "act(gate) * up");
+  m.def("sigmoid_topk_route", &sigmoid_topk_route, "sigmoid top-k router");
+  m.def("routed_scaled_silu_mul", &routed_scaled_silu_mul,
+        "stacked-expert SiLU with input-side routing weight");
+}
