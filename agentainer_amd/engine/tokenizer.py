@@ -17,13 +17,16 @@ MIN_VOCAB = 256 + OFFSET
 
 class ByteTokenizer:
     def __init__(self, vocab_size: int):
-        assert vocab_size >= MIN_VOCAB, f"vocab must be >= {MIN_VOCAB}"
+        # a checkpoint with fewer ids than bytes still serves: bytes fold
+        # onto the ids it has (lossy text, valid ids)
+        assert vocab_size > OFFSET, f"vocab must be > {OFFSET}"
         self.vocab_size = vocab_size
+        self._span = min(256, vocab_size - OFFSET)
         self.eos_id = EOS
         self.bos_id = BOS
 
     def encode(self, text: str, bos: bool = False) -> List[int]:
-        ids = [b + OFFSET for b in text.encode("utf-8")]
+        ids = [b % self._span + OFFSET for b in text.encode("utf-8")]
         return ([BOS] if bos else []) + ids
 
     def decode(self, ids: List[int]) -> str:
