@@ -233,7 +233,7 @@ class GatedFeedForward(torch.nn.Module):
         self.gate_up.copy_(torch.cat([get("gate"), get("up")], dim=0))
         self.down.copy_(get("down"))
 
-    def forward(self, h):
+    def forward(self, h, allow_gather: bool = True):
         gu = ops.linear(h, self.gate_up)
         act = torch.empty(h.size(0), self.ff, dtype=h.dtype, device=h.device)
         ops.act_mul(act, gu[:, :self.ff], gu[:, self.ff:], self.act)
@@ -272,12 +272,15 @@ class SigmoidRoutedExperts(torch.nn.Module):
         self.down.copy_(torch.cat([get(f"e{e}.down") for e in range(E)],
                                   dim=1))
 
-    def forward(self, h):
+    def forward(self, h, allow_gather: bool = True):
+        """allow_gather=False keeps the step free of host syncs (decode
+        steps are captured into a hipGraph)."""
         T = h.size(0)
         logits = F.linear(h.float(), self.router)              # fp32 router
         weight = torch.empty(T, self.E, dtype=torch.float32, device=h.device)
         ops.sigmoid_topk_route(weight, logits, self.top)
-        if T >= self.SPARSE_MIN_TOKENS and self.E > self.top:
+        if (allow_gather and T >= self.SPARSE_MIN_TOKENS
+                and self.E > self.top):
             return self._gathered(h, weight)
         gu = ops.linear(h, self.gate_up)                       # [T, E*2F]
         act = torch.empty(T, self.E * self.ff, dtype=h.dtype, device=h.device)
@@ -438,7 +441,8 @@ class LelitarForCausalLM(torch.nn.Module):
             if isinstance(cache, (tuple, list)):
                 cache = cache[0]
             y_mix = layer.mix(hs[0], cache, md)
-            y_ff = layer.mlp(hs[1]) if layer.mlp is not None else None
+            y_ff = (layer.mlp(hs[1], allow_gather=md.is_prefill)
+                    if layer.mlp is not None else None)
             nxt = (self.layers[i + 1].norm_weights() if i + 1 < n
                    else [self.final_norm])
             hs = norms(y_mix, y_ff, nxt)

@@ -181,7 +181,8 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(
     long q_ts, long o_hs, long o_ts, const short* __restrict__ cache,
     const int* __restrict__ page_table, const int* __restrict__ seq_lens,
     const int* __restrict__ q_starts, const int* __restrict__ q_lens,
-    float scale, int window, int H, int nc, int PS, int max_pages) {
+    float scale, int window, int H, int nc, int PS, int max_pages,
+    float* __restrict__ part_o, float* __restrict__ part_ml, int n_splits) {
   extern __shared__ __attribute__((aligned(16))) short lds[];
   const int Rp = nc * 32;
   const int KS = Rp + 8;                       // padded row-major stride
@@ -201,6 +202,7 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(
   const int l16 = lane % 16, lg = lane / 16;
 
   if (total <= 0) {  // pad row of a captured decode batch: zeros
+    if (n_splits > 0) return;  // the combine kernel writes them
     for (int i = threadIdx.x; i < nrows * Rp; i += 256) {
       const int r = i / Rp, d = i % Rp;
       out[(r % H) * o_hs + (row_base + r / H) * o_ts + d] = 0;
@@ -212,8 +214,16 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(
 
   // block's key span: first row's window start .. last row's position
   const int r_last = min(r0 + ROWS_PER_BLOCK, nrows) - 1;
-  const int kv_lo = max(0, ctx + r0 / H - window + 1);
-  const int kv_hi = ctx + r_last / H;  // inclusive
+  int kv_lo = max(0, ctx + r0 / H - window + 1);
+  int kv_hi = ctx + r_last / H;  // inclusive
+  if (n_splits > 0) {
+    // split-KV (decode): this block owns one 32-aligned slice of the span;
+    // an empty slice still writes its (m = -max, l = 0) partial below
+    const int n_keys = kv_hi - kv_lo + 1;
+    const int span = ((n_keys + n_splits - 1) / n_splits + KVT - 1) / KVT * KVT;
+    kv_lo += blockIdx.z * span;
+    kv_hi = min(kv_hi, kv_lo + span - 1);
+  }
 
   // ---- this wave's Q fragments: lane -> row l16, cols dc*32 + lg*8..+8
   const int rw0 = r0 + wid * ROWS_PER_WAVE;
@@ -293,7 +303,7 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(
 #pragma unroll
         for (int ks = 0; ks < 2; ++ks) {
           const int kpos = kv0 + ks * 16 + l16;
-          const bool seen = rok[r] && kpos <= qpos[r] &&
+          const bool seen = rok[r] && kpos <= qpos[r] && kpos <= kv_hi &&
                             qpos[r] - kpos < window;
           s[ks][r] = seen ? s[ks][r] * scale : -FLT_MAX;
         }
@@ -342,6 +352,22 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(
   }
 
   // ---- epilogue
+  if (n_splits > 0) {  // unnormalized partials (rows are heads: qlen == 1)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int rr = rw0 + lg * 4 + r;
+      if (rr >= nrows) continue;
+      const long pr = ((long)b * n_splits + blockIdx.z) * H + rr;
+      if (l16 == 0) {
+        part_ml[pr * 2] = m_run[r];
+        part_ml[pr * 2 + 1] = l_run[r];
+      }
+#pragma unroll
+      for (int dt = 0; dt < 2 * MAXNC; ++dt)
+        if (dt < 2 * nc) part_o[pr * Rp + dt * 16 + l16] = o[dt][r];
+    }
+    return;
+  }
 #pragma unroll
   for (int r = 0; r < 4; ++r) {
     const int rr = rw0 + lg * 4 + r;
@@ -354,18 +380,63 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(
   }
 }
 
-template <typename T>
+// merge the split-KV partials of one (sequence, head): log-sum-exp rescale
+__global__ __launch_bounds__(64) void latent_attn_combine_kernel(
+    short* __restrict__ out, long o_hs, long o_ts,
+    const float* __restrict__ part_o, const float* __restrict__ part_ml,
+    const int* __restrict__ seq_lens, int H, int Rp, int n_splits) {
+  const int h = blockIdx.x, b = blockIdx.y;
+  short* op = out + h * o_hs + (long)b * o_ts;
+  if (seq_lens[b] <= 0) {
+    for (int d = threadIdx.x; d < Rp; d += WAVE) op[d] = 0;
+    return;
+  }
+  float M = -FLT_MAX;
+  for (int s = 0; s < n_splits; ++s)
+    M = fmaxf(M, part_ml[(((long)b * n_splits + s) * H + h) * 2]);
+  float L = 0.f;
+  for (int s = 0; s < n_splits; ++s) {
+    const long pr = ((long)b * n_splits + s) * H + h;
+    const float m = part_ml[pr * 2];
+    if (m != -FLT_MAX) L += part_ml[pr * 2 + 1] * __expf(m - M);
+  }
+  const float inv = L > 0.f ? 1.0f / L : 0.f;
+  for (int d = threadIdx.x; d < Rp; d += WAVE) {
+    float acc = 0.f;
+    for (int s = 0; s < n_splits; ++s) {
+      const long pr = ((long)b * n_splits + s) * H + h;
+      const float m = part_ml[pr * 2];
+      if (m != -FLT_MAX) acc += part_o[pr * Rp + d] * __expf(m - M);
+    }
+    op[d] = f2bits(acc * inv);
+  }
+}
+
+template <typename T, int VEC>
 __global__ void sigmoid_gate_mul_kernel(T* __restrict__ out,
                                         const T* __restrict__ a, long a_hs,
                                         long a_ts, const T* __restrict__ g,
                                         long g_rs, long n, int H, int E) {
-  const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  const long i = ((long)blockIdx.x * blockDim.x + threadIdx.x) * VEC;
   if (i >= n) return;
   const long t = i / ((long)H * E);
   const int c = (int)(i % ((long)H * E));
   const int h = c / E, e = c % E;
-  const float gv = ldf(g, t * g_rs + c);
-  stf(out, i, ldf(a, h * a_hs + t * a_ts + e) / (1.0f + expf(-gv)));
+  float gv[VEC], av[VEC], o[VEC];
+  if constexpr (VEC == 4) {
+    ld4(g, t * g_rs + c, gv);
+    ld4(a, h * a_hs + t * a_ts + e, av);
+  } else {
+    gv[0] = ldf(g, t * g_rs + c);
+    av[0] = ldf(a, h * a_hs + t * a_ts + e);
+  }
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) o[j] = av[j] / (1.0f + expf(-gv[j]));
+  if constexpr (VEC == 4) {
+    st4(out, i, o);
+  } else {
+    stf(out, i, o[0]);
+  }
 }
 
 size_t mfma_lds_bytes(int Rp) {
@@ -455,7 +526,23 @@ void latent_window_attention(torch::Tensor out, torch::Tensor q_lat,
     const int nc = Rp / 32;
     const size_t lds = mfma_lds_bytes(Rp);
     const long rows = max_qlen * H;
-    dim3 grid((rows + ROWS_PER_BLOCK - 1) / ROWS_PER_BLOCK, B);
+    const int row_blocks = (rows + ROWS_PER_BLOCK - 1) / ROWS_PER_BLOCK;
+    // decode: too few (sequence, row-block) pairs to fill 256 CUs — cut
+    // every sequence's key span into slices (>= 64 keys each) and merge
+    int n_splits = 0;
+    torch::Tensor part_o, part_ml;
+    if (!query_starts.has_value()) {
+      const long n_max = std::min<long>(window, (long)max_pages * PS);
+      const long want = (512 + (long)B * row_blocks - 1) / ((long)B * row_blocks);
+      const long s = std::min<long>(want, n_max / 64);
+      if (s >= 2) {
+        n_splits = (int)s;
+        auto fo = torch::TensorOptions().dtype(torch::kFloat).device(out.device());
+        part_o = torch::empty({(long)B * n_splits * H * Rp}, fo);
+        part_ml = torch::empty({(long)B * n_splits * H * 2}, fo);
+      }
+    }
+    dim3 grid(row_blocks, B, n_splits > 0 ? n_splits : 1);
     bool launched = true;
 #define LA_LAUNCH(MAXNC)                                                       \
   do {                                                                         \
@@ -476,13 +563,22 @@ void latent_window_attention(torch::Tensor out, torch::Tensor q_lat,
                        (const short*)cache.data_ptr(),                         \
                        page_table.data_ptr<int>(), seq_lens.data_ptr<int>(),   \
                        qs, ql, (float)scale, (int)window, H, nc, PS,           \
-                       max_pages);                                             \
+                       max_pages,                                              \
+                       n_splits > 0 ? part_o.data_ptr<float>() : nullptr,      \
+                       n_splits > 0 ? part_ml.data_ptr<float>() : nullptr,     \
+                       n_splits);                                              \
   } while (0)
     if (nc <= 2) LA_LAUNCH(2);
     else if (nc <= 4) LA_LAUNCH(4);
     else if (nc <= 8) LA_LAUNCH(8);
     else LA_LAUNCH(16);
 #undef LA_LAUNCH
+    if (launched && n_splits > 0)
+      hipLaunchKernelGGL(latent_attn_combine_kernel, dim3(H, B), dim3(64), 0,
+                         stream, (short*)out.data_ptr(), (long)out.stride(0),
+                         (long)out.stride(1), part_o.data_ptr<float>(),
+                         part_ml.data_ptr<float>(), seq_lens.data_ptr<int>(),
+                         H, Rp, n_splits);
     if (launched) return;
   }
   TORCH_CHECK(Rp <= WAVE * RW_MAX_ACC, "latent rank too large");
@@ -509,12 +605,23 @@ void sigmoid_gate_mul(torch::Tensor out, torch::Tensor a, torch::Tensor g) {
   TORCH_CHECK(g.size(0) == T_ && g.size(1) == (long)H * E);
   const long n = (long)T_ * H * E;
   if (n == 0) return;
+  const bool vec = E % 4 == 0 && a.stride(0) % 4 == 0 && a.stride(1) % 4 == 0 &&
+                   a.storage_offset() % 4 == 0 && g.stride(0) % 4 == 0 &&
+                   g.storage_offset() % 4 == 0;
   auto stream = at::hip::getCurrentHIPStream();
   LATENT_DISPATCH_T(out, {
-    hipLaunchKernelGGL(sigmoid_gate_mul_kernel<T>, dim3((n + 255) / 256),
-                       dim3(256), 0, stream, (T*)out.data_ptr(),
-                       (const T*)a.data_ptr(), (long)a.stride(0),
-                       (long)a.stride(1), (const T*)g.data_ptr(),
-                       (long)g.stride(0), n, H, E);
+    if (vec) {
+      hipLaunchKernelGGL((sigmoid_gate_mul_kernel<T, 4>),
+                         dim3((n / 4 + 255) / 256), dim3(256), 0, stream,
+                         (T*)out.data_ptr(), (const T*)a.data_ptr(),
+                         (long)a.stride(0), (long)a.stride(1),
+                         (const T*)g.data_ptr(), (long)g.stride(0), n, H, E);
+    } else {
+      hipLaunchKernelGGL((sigmoid_gate_mul_kernel<T, 1>),
+                         dim3((n + 255) / 256), dim3(256), 0, stream,
+                         (T*)out.data_ptr(), (const T*)a.data_ptr(),
+                         (long)a.stride(0), (long)a.stride(1),
+                         (const T*)g.data_ptr(), (long)g.stride(0), n, H, E);
+    }
   });
 }

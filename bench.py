@@ -50,6 +50,10 @@ from agentainer_amd.wal import RequestManager
 
 
 def parse_args():
+    return _parser().parse_args()
+
+
+def _parser():
     p = argparse.ArgumentParser()
     p.add_argument("--gpus", type=int, default=1)
     p.add_argument("--steps", type=int, default=300)
@@ -73,7 +77,140 @@ def parse_args():
     p.add_argument("--dense-quant", default="", choices=["", "fp8", "mxfp4"],
                    help="opt-in quantized dense decode projections (turbo; "
                         "NOT the headline dtype)")
-    return p.parse_args()
+    p.add_argument("--arch-compare", action="store_true",
+                   help="instead of the headline workload: prefill and decode "
+                        "tokens/s of the Lelitar design at real-layer sizes "
+                        "beside Llama/Mixtral stacks of equal size")
+    p.add_argument("--arch-sizes", default="s,l,moe",
+                   help="--arch-compare: which size points to run")
+    return p
+
+
+def _arch_points():
+    """Size points: (name, Lelitar config, reference model config, class).
+    A few layers each — throughput per layer is what is compared."""
+    from agentainer_amd.models.lelitar import (FeedForwardConfig,
+                                               LatentMixerConfig,
+                                               LelitarConfig,
+                                               LelitarLayerConfig)
+    from agentainer_amd.models.llama import LlamaConfig
+    from agentainer_amd.models.mixtral import MixtralConfig
+
+    def lel(name, width, heads, q_rank, kv_rank, window, ff, n, moe=None):
+        mlp = (FeedForwardConfig("moe", ff, experts=moe[0], top=moe[1])
+               if moe else FeedForwardConfig("dense", ff))
+        mixer = LatentMixerConfig(heads=heads, dim=128, vdim=128,
+                                  q_rank=q_rank, kv_rank=kv_rank,
+                                  window=window, scale=128 ** -0.5)
+        return LelitarConfig(name=name, vocab_size=32000, hidden_size=width,
+                             layers=[LelitarLayerConfig(mixer, mlp)
+                                     for _ in range(n)],
+                             norm_eps=1e-6, norm_groups=2, residual_mult=0.5)
+
+    pts = {
+        "s": ("w2048-ff8192", lel("lelitar-s", 2048, 16, 768, 256, 1024,
+                                  8192, 4),
+              LlamaConfig(name="llama-s", vocab_size=32000, hidden_size=2048,
+                          n_layers=4, n_heads=16, n_kv_heads=4,
+                          intermediate_size=8192, tie_embeddings=False), None),
+        "l": ("w4096-ff14336", lel("lelitar-l", 4096, 32, 1536, 512, 4096,
+                                   14336, 4),
+              LlamaConfig(name="llama-l", vocab_size=32000, hidden_size=4096,
+                          n_layers=4, n_heads=32, n_kv_heads=8,
+                          intermediate_size=14336, tie_embeddings=False),
+              None),
+        "moe": ("w2048-8x4096-top2", lel("lelitar-moe", 2048, 16, 768, 256,
+                                         1024, 4096, 4, moe=(8, 2)),
+                MixtralConfig(name="mixtral-s", vocab_size=32000,
+                              hidden_size=2048, n_layers=4, n_heads=16,
+                              n_kv_heads=4, intermediate_size=4096,
+                              n_experts=8, top_k=2, tie_embeddings=False),
+                "mixtral"),
+    }
+    return pts
+
+
+def run_arch_compare(args):
+    """Prefill (8 x 1024-token prompts per step) and decode (64 sequences at
+    1024 tokens of context, captured graph) throughput, through the
+    engine's own varlen and decode step functions."""
+    from agentainer_amd.engine.llm import ModelInstance
+    from agentainer_amd.models.lelitar import LelitarForCausalLM
+    from agentainer_amd.models.mixtral import MixtralForCausalLM
+
+    dev = "cuda" if torch.cuda.is_available() else "cpu"
+    small = dev == "cpu"
+    n_pf, pf_len, n_dec, ctx = (2, 64, 4, 64) if small else (8, 1024, 64, 1024)
+    steps = max(3, min(args.steps, 20))
+    ecfg = {"sync_mode": True, "async_decode": False, "prefill_stream": False,
+            "prefix_sharing": False, "kv_page_size": 16,
+            "kv_pool_tokens": (n_dec + n_pf) * (ctx + 256) + 4096,
+            "max_seqs": n_dec + n_pf + 2, "max_batch_tokens": 1 << 20,
+            "max_decode_batch": n_dec}
+
+    def sync():
+        if dev == "cuda":
+            torch.cuda.synchronize()
+
+    def measure(name, cfg, cls):
+        inst = ModelInstance(name, cfg, dev, ecfg, model_cls=cls)
+        g = torch.Generator().manual_seed(0)
+
+        def toks(n):
+            return torch.randint(3, cfg.vocab_size, (n,), generator=g).tolist()
+
+        # prefill: fresh sequences every step
+        pf_ms = []
+        for it in range(steps + 2):
+            plan = [(f"p{i}", toks(pf_len), False, None) for i in range(n_pf)]
+            sync()
+            t0 = time.time()
+            inst._prefill_exec(plan)
+            sync()
+            if it >= 2:
+                pf_ms.append((time.time() - t0) * 1e3)
+            for i in range(n_pf):
+                inst.kvm.free_seq(f"p{i}")
+        # decode: n_dec sequences with ctx tokens of context
+        for i in range(0, n_dec, 8):
+            inst._prefill_exec([(f"d{j}", toks(ctx), False, None)
+                                for j in range(i, min(i + 8, n_dec))])
+        plan = [(f"d{j}", 5) for j in range(n_dec)]
+        dec_ms = []
+        for it in range(steps * 4 + 4):
+            sync()
+            t0 = time.time()
+            inst._decode_exec(plan)
+            sync()
+            if it >= 4:
+                dec_ms.append((time.time() - t0) * 1e3)
+        del inst
+        if dev == "cuda":
+            torch.cuda.empty_cache()
+        pf = statistics.median(pf_ms)
+        dc = statistics.median(dec_ms)
+        return {"prefill_ms": round(pf, 3),
+                "prefill_tok_s": round(n_pf * pf_len / pf * 1e3),
+                "decode_ms": round(dc, 3),
+                "decode_tok_s": round(n_dec / dc * 1e3)}
+
+    pts = _arch_points()
+    for key in args.arch_sizes.split(","):
+        label, lcfg, rcfg, kind = pts[key.strip()]
+        if small:  # CPU dry run: shrink to something that finishes
+            continue
+        ours = measure(lcfg.name, lcfg, LelitarForCausalLM)
+        theirs = measure(rcfg.name, rcfg,
+                         MixtralForCausalLM if kind == "mixtral" else None)
+        print(json.dumps({
+            "metric": "arch_compare", "point": label, "layers": rcfg.n_layers,
+            "prefill": f"{n_pf}x{pf_len}", "decode": f"{n_dec}@{ctx}",
+            "dtype": "bf16", "data": "synthetic", "lelitar": ours,
+            "reference_model": rcfg.name, "reference": theirs,
+            "prefill_ratio": round(ours["prefill_tok_s"]
+                                   / theirs["prefill_tok_s"], 3),
+            "decode_ratio": round(ours["decode_tok_s"]
+                                  / theirs["decode_tok_s"], 3)}), flush=True)
 
 
 class ClosedLoopClient:
@@ -133,6 +270,9 @@ class ClosedLoopClient:
 
 def main():
     args = parse_args()
+    if args.arch_compare:
+        run_arch_compare(args)
+        return
     rank = int(os.environ.get("RANK", "0"))
     world = int(os.environ.get("WORLD_SIZE", "1"))
     has_gpu = torch.cuda.is_available()

@@ -131,16 +131,26 @@ def test_latent_attention_varlen_fp32(H, Rp, PS, window):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
-def test_latent_attention_decode_rows(dtype):
+@pytest.mark.parametrize("H,window,lens", [
+    (4, 20, [37, 0, 1, 64]),
+    (4, 200, [300, 0, 1, 130, 64, 257]),       # key span cut into slices
+    (70, 1000, [640, 33, 0, 129])])            # heads span two row blocks
+def test_latent_attention_decode_rows(dtype, H, window, lens):
     """Decode form: no query_starts/lens; a row with seq_len <= 0 is a pad
     row and must come back as zeros."""
     g = torch.Generator().manual_seed(5)
-    H, Rp, PS, window = 4, 64, 16, 20
-    seq = torch.tensor([37, 0, 1, 64], dtype=torch.int32)
-    B = 4
-    cache = (torch.randn(16, PS, Rp, generator=g) * 0.7).to(dtype)
-    pt = torch.tensor([[1, 2, 3, 0], [0, 0, 0, 0], [4, 0, 0, 0],
-                       [5, 6, 7, 8]], dtype=torch.int32)
+    Rp, PS = 64, 16
+    seq = torch.tensor(lens, dtype=torch.int32)
+    B = len(lens)
+    width = max(-(-n // PS) for n in lens)
+    n_pages = sum(-(-n // PS) for n in lens) + 1
+    cache = (torch.randn(n_pages, PS, Rp, generator=g) * 0.7).to(dtype)
+    perm = (torch.randperm(n_pages - 1, generator=g) + 1).tolist()
+    pt = torch.zeros(B, width, dtype=torch.int32)
+    for b, n in enumerate(lens):
+        k = -(-n // PS)
+        pt[b, :k] = torch.tensor([perm.pop() for _ in range(k)],
+                                 dtype=torch.int32)
     q = (torch.randn(H, B, Rp, generator=g) * 0.5).to(dtype)
     out_r = torch.ones(H, B, Rp, dtype=dtype)
     ref.latent_window_attention(out_r, q, cache, pt, seq, None, None, 0.2,
@@ -148,7 +158,7 @@ def test_latent_attention_decode_rows(dtype):
     out_d = torch.ones(H, B, Rp, dtype=dtype, device="cuda")
     ops.latent_window_attention(out_d, q.cuda(), cache.cuda(), pt.cuda(),
                                 seq.cuda(), None, None, 0.2, window)
-    assert float(out_d[:, 1].abs().max()) == 0.0
+    assert float(out_d[:, lens.index(0)].abs().max()) == 0.0
     torch.testing.assert_close(out_d.cpu().float(), out_r.float(),
                                **_tol(dtype))
 

@@ -75,6 +75,9 @@ BEACON_CASES = [
     (64, 8, 20, 20, 19, 19),   # the very first token, window > sequence
     (33, 8, 70, 70, 40, 32),   # inside, whole prompt in one portion
     (33, 8, 70, 70, 40, 33),   # outside
+    (150, 16, 400, 1, 0, 149),  # decoded, span cut into key slices: inside
+    (150, 16, 400, 1, 0, 150),  # ... and just outside
+    (300, 16, 700, 1, 0, 0),    # decoded, many slices, beacon is the token
     (1, 4, 9, 3, 1, 0),        # window of one: only itself
     (1, 4, 9, 3, 1, 1),
 ]
