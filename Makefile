@@ -4,7 +4,7 @@ PY ?= python
 .PHONY: build build-asan install test test-gpu test-gpu-serialized test-sanitize test-crash test-persistence test-network test-all bench verify
 
 build:
-	$(PY) -m agentainer_amd.ops.build
+	$(PY) -m agentainer_amd.ops.build all
 
 # host-AddressSanitized binding layer (SURVEY.md §5 sanitizer row);
 # run via LD_PRELOAD=$$(hipcc -print-file-name=libclang_rt.asan-x86_64.so)

@@ -466,6 +466,8 @@ def latent_norm_append(proj, q_off, q_rank, kv_off, kv_rank, wq, wkv, eps,
 # AGENTAINER_LATENT_SIMPLE=1 forces the one-wave-per-row kernel (A/B and
 # numerics cross-checks against the MFMA tile kernel)
 LATENT_SIMPLE = os.environ.get("AGENTAINER_LATENT_SIMPLE", "0") == "1"
+# decode key-span slices per sequence; 0 = sized to fill the chip
+LATENT_SPLITS = int(os.environ.get("AGENTAINER_LATENT_SPLITS", "0"))
 
 
 def latent_window_attention(out, q_lat, cache, page_table, seq_lens,
@@ -476,7 +478,7 @@ def latent_window_attention(out, q_lat, cache, page_table, seq_lens,
         mod.latent_window_attention(out, q_lat, cache, page_table, seq_lens,
                                     query_starts, query_lens, float(scale),
                                     int(window), int(max_qlen),
-                                    bool(LATENT_SIMPLE))
+                                    bool(LATENT_SIMPLE), int(LATENT_SPLITS))
     else:
         reference.latent_window_attention(out, q_lat, cache, page_table,
                                           seq_lens, query_starts, query_lens,

@@ -263,23 +263,51 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(
 #pragma unroll
   for (int r = 0; r < 4; ++r) { m_run[r] = -FLT_MAX; l_run[r] = 0.f; }
 
-  const int chunks_per_tok = Rp / 8;
-  const int n_chunks = KVT * chunks_per_tok;
-
-  for (int kv0 = kv_lo; kv0 <= kv_hi; kv0 += KVT) {
-    // ---- stage the tile: row-major (K role) + transposed (V role)
-    for (int c = threadIdx.x; c < n_chunks; c += 256) {
-      const int tok = c / chunks_per_tok, d8 = c % chunks_per_tok;
-      const int gt = kv0 + tok;
-      bf16x8 v{};
-      if (gt <= kv_hi)
-        v = *reinterpret_cast<const bf16x8*>(
-            cache + ((long)pt[gt / PS] * PS + gt % PS) * Rp + d8 * 8);
-      *reinterpret_cast<bf16x8*>(k_lds + tok * KS + d8 * 8) = v;
+  const int n_chunks = KVT * (Rp / 8);
+  // Staging is split in two so that a whole tile's global loads are in
+  // flight at once and overlap the previous tile's MFMAs: stage_load
+  // issues every 16-B load of the NEXT tile into registers, stage_write
+  // (after the barrier that retires the current tile's readers) stores
+  // them row-major (K role) and transposed (V role).
+  // chunk -> (token fast, 16-B column slow): the transposed 2-byte writes
+  // of one wave land on consecutive LDS addresses (a column-fast mapping
+  // puts all 64 lanes on two banks), and the block's 4 waves together
+  // consume whole 128-B lines of each row.
+  constexpr int MAXIT = (MAXNC + 1) / 2;  // ceil(n_chunks / 256)
+  bf16x8 st[MAXIT];
+  auto stage_load = [&](int kv0) {
 #pragma unroll
-      for (int j = 0; j < 8; ++j) vt_lds[(d8 * 8 + j) * VT_STRIDE + tok] = v[j];
+    for (int k = 0; k < MAXIT; ++k) {
+      const int c = threadIdx.x + 256 * k;
+      st[k] = bf16x8{};
+      if (c < n_chunks) {
+        const int tok = c % KVT, d8 = c / KVT;
+        const int gt = kv0 + tok;
+        if (gt <= kv_hi)
+          st[k] = *reinterpret_cast<const bf16x8*>(
+              cache + ((long)pt[gt / PS] * PS + gt % PS) * Rp + d8 * 8);
+      }
     }
+  };
+  auto stage_write = [&]() {
+#pragma unroll
+    for (int k = 0; k < MAXIT; ++k) {
+      const int c = threadIdx.x + 256 * k;
+      if (c < n_chunks) {
+        const int tok = c % KVT, d8 = c / KVT;
+        *reinterpret_cast<bf16x8*>(k_lds + tok * KS + d8 * 8) = st[k];
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+          vt_lds[(d8 * 8 + j) * VT_STRIDE + tok] = st[k][j];
+      }
+    }
+  };
+
+  if (kv_lo <= kv_hi) stage_load(kv_lo);
+  for (int kv0 = kv_lo; kv0 <= kv_hi; kv0 += KVT) {
+    stage_write();
     __syncthreads();
+    if (kv0 + KVT <= kv_hi) stage_load(kv0 + KVT);
 
     if (wave_live && kv0 <= w_hi && kv0 + KVT > w_lo) {
       // ---- S = Q K^T, two 16-key sub-tiles
@@ -333,7 +361,9 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(
 #pragma unroll
         for (int r = 0; r < 4; ++r)
           pw[(lg * 4 + r) * P_STRIDE + ks * 16 + l16] = f2bits(s[ks][r]);
-      __builtin_amdgcn_s_waitcnt(0);  // own-wave LDS ordering
+      // own-wave LDS ordering: wait for LDS traffic only (lgkmcnt = 0),
+      // the next tile's global loads stay in flight
+      __builtin_amdgcn_s_waitcnt(0xc07f);
       const bf16v8 pf =
           *reinterpret_cast<const bf16v8*>(pw + l16 * P_STRIDE + lg * 8);
       // ---- O = alpha O + P V
@@ -485,7 +515,7 @@ void latent_window_attention(torch::Tensor out, torch::Tensor q_lat,
                              c10::optional<torch::Tensor> query_starts,
                              c10::optional<torch::Tensor> query_lens,
                              double scale, long window, long max_qlen,
-                             bool force_simple) {
+                             bool force_simple, long splits) {
   TORCH_CHECK(q_lat.dim() == 3 && out.dim() == 3 && q_lat.stride(2) == 1 &&
               out.stride(2) == 1);
   TORCH_CHECK(cache.dim() == 3 && cache.is_contiguous());
@@ -533,8 +563,10 @@ void latent_window_attention(torch::Tensor out, torch::Tensor q_lat,
     torch::Tensor part_o, part_ml;
     if (!query_starts.has_value()) {
       const long n_max = std::min<long>(window, (long)max_pages * PS);
-      const long want = (512 + (long)B * row_blocks - 1) / ((long)B * row_blocks);
-      const long s = std::min<long>(want, n_max / 64);
+      // one resident workgroup per CU at large ranks: aim at one wave of
+      // 256 workgroups — more slices only add partial-merge traffic
+      const long want = (256 + (long)B * row_blocks - 1) / ((long)B * row_blocks);
+      const long s = splits > 0 ? splits : std::min<long>(want, n_max / 64);
       if (s >= 2) {
         n_splits = (int)s;
         auto fo = torch::TensorOptions().dtype(torch::kFloat).device(out.device());

@@ -17,7 +17,7 @@ void latent_window_attention(torch::Tensor out, torch::Tensor q_lat,
                              c10::optional<torch::Tensor> query_starts,
                              c10::optional<torch::Tensor> query_lens,
                              double scale, long window, long max_qlen,
-                             bool force_simple);
+                             bool force_simple, long splits);
 void sigmoid_gate_mul(torch::Tensor out, torch::Tensor a, torch::Tensor g);
 void act_mul(torch::Tensor out, torch::Tensor gate, torch::Tensor up, long act);
 void sigmoid_topk_route(torch::Tensor weight, torch::Tensor logits, long top);
