@@ -995,6 +995,13 @@ class ModelInstance:
         for seq_id, _toks in entries:
             if not self.kvm.has_seq(seq_id):
                 self._bind_seq(seq_id, None)
+        # an entry that brings no tokens only admits its sequence
+        live = [i for i, (_s, t) in enumerate(entries) if len(t) > 0]
+        if len(live) < len(entries):
+            entries = [entries[i] for i in live]
+            want = [want[i] for i in live]
+        if not entries:
+            return torch.empty(0, self.cfg.vocab_size, device=self.device)
         decode = all(len(t) == 1 and self.kvm.seq_len(s) > 0
                      for s, t in entries)
         if decode and len(entries) <= max(self.max_decode_batch, 1):

@@ -265,14 +265,20 @@ def test_greedy_generation_through_scheduler(tmp_path, device):
 
 
 @pytest.mark.gpu
-def test_bf16_serving_path_close_to_oracle(tmp_path):
+@pytest.mark.parametrize("shape", [
+    dict(width=128, heads=4, dim=32, vdim=32, q_rank=64, kv_rank=64,
+         window=40, ff=256, expert_ff=64, experts=4, top=2),
+    # nothing a multiple of 32, rank padded inside the pool
+    dict(width=48, heads=3, dim=8, vdim=20, q_rank=24, kv_rank=40, groups=3,
+         window=23, ff=56, expert_ff=12, experts=7, top=3),
+    dict(width=72, heads=5, dim=24, vdim=8, q_rank=40, kv_rank=136, groups=1,
+         window=130, ff=40, expert_ff=20, experts=3, top=1)])
+def test_bf16_serving_path_close_to_oracle(tmp_path, shape):
     """bf16 serving precision (MFMA tile attention, captured decode graph):
     logits stay within bf16 rounding of the fp32 oracle, and graph replays
     keep agreeing with it step after step."""
-    cfg = O.random_config(width=128, heads=4, dim=32, vdim=32, q_rank=64,
-                          kv_rank=64, window=40, ff=256, expert_ff=64,
-                          experts=4, top=2, vocab=300, n_layers=4,
-                          kinds=("dense", "moe"))
+    cfg = O.random_config(vocab=300, n_layers=4, kinds=("dense", "moe"),
+                          **shape)
     w = O.random_weights(cfg, seed=11, std=0.2)
     eng, inst, _ = make_instance(tmp_path, cfg, w, "cuda", dtype="bfloat16",
                                  page=16, pool_tokens=512)
