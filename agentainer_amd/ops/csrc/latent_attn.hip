@@ -410,15 +410,215 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(
   }
 }
 
+// ------------------------------------------------------------------
+// latent_decode_mfma: decode (one new token per sequence), bf16.
+//
+// The tile kernel above keeps a whole [16 x Rp] fp32 accumulator per wave,
+// which at large ranks leaves one barrier-bound workgroup per CU. Here the
+// RANK is split over the 4 waves of a workgroup instead: wave w owns
+// columns [w*Rp/4, (w+1)*Rp/4) of every key row — for the QK^T contraction
+// (partial scores, summed across the waves through LDS) and as its slice of
+// the output. Each wave loads its quarter of 32 key rows straight from
+// global memory into MFMA B-fragments, transposes the same registers
+// through a private LDS patch for the PV product, and keeps only
+// [16 x Rp/4] accumulators, so several workgroups share a CU and hide one
+// another's load latency. One barrier per 32-key tile (score exchange is
+// double-buffered). grid = (sequence, key slice, 16-head row tile);
+// results are unnormalized partials for latent_attn_combine.
+// ------------------------------------------------------------------
+template <int NCW>  // 32-wide rank chunks per wave: Rp = 128 * NCW
+__global__ __launch_bounds__(256) void latent_decode_mfma_kernel(
+    float* __restrict__ part_o, float* __restrict__ part_ml,
+    const short* __restrict__ q_lat, long q_hs, long q_ts,
+    const short* __restrict__ cache, const int* __restrict__ page_table,
+    const int* __restrict__ seq_lens, float scale, int window, int H, int PS,
+    int max_pages, int n_splits) {
+  constexpr int CW = NCW * 32;   // columns per wave
+  constexpr int Rp = CW * 4;
+  constexpr int NDT = CW / 16;   // 16-wide output tiles per wave
+  constexpr int S_STRIDE = KVT + 1;
+  __shared__ __attribute__((aligned(16))) short vt_lds[4][CW * VT_STRIDE];
+  __shared__ __attribute__((aligned(16))) short p_lds[4][16 * P_STRIDE];
+  __shared__ float s_lds[2][4][16 * S_STRIDE];
+
+  const int b = blockIdx.x, split = blockIdx.y, rt = blockIdx.z;
+  const int total = seq_lens[b];
+  if (total <= 0) return;  // pad row: the combine kernel writes zeros
+  const int lane = threadIdx.x % WAVE, wid = threadIdx.x / WAVE;
+  const int l16 = lane % 16, lg = lane / 16;
+  const int col0 = wid * CW;
+  const int* pt = page_table + (long)b * max_pages;
+
+  const int qpos = total - 1;
+  int kv_lo = max(0, qpos - window + 1);
+  int kv_hi = qpos;
+  {
+    const int n_keys = kv_hi - kv_lo + 1;
+    const int span = ((n_keys + n_splits - 1) / n_splits + KVT - 1) / KVT * KVT;
+    kv_lo += split * span;
+    kv_hi = min(kv_hi, kv_lo + span - 1);
+  }
+
+  // Q fragments (A operand): row = head rt*16 + l16, this wave's columns
+  bf16v8 qf[NCW];
+  {
+    const int h = rt * 16 + l16;
+    const short* qp = q_lat + (long)min(h, H - 1) * q_hs + (long)b * q_ts + col0;
+#pragma unroll
+    for (int dc = 0; dc < NCW; ++dc)
+      qf[dc] = h < H ? *reinterpret_cast<const bf16v8*>(qp + dc * 32 + lg * 8)
+                     : bf16v8{};
+  }
+  f32x4 o[NDT];
+#pragma unroll
+  for (int dt = 0; dt < NDT; ++dt) o[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  float m_run[4], l_run[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) { m_run[r] = -FLT_MAX; l_run[r] = 0.f; }
+
+  // page ids are looked up TWO tiles ahead and rows ONE tile ahead, so the
+  // dependent (page table -> row) load chain never sits on the critical path
+  auto pages_of = [&](int kv0, int (&pg)[2]) {
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+      const int key = kv0 + ks * 16 + l16;
+      pg[ks] = key <= kv_hi ? pt[key / PS] : -1;
+    }
+  };
+  auto load_tile = [&](int kv0, const int (&pg)[2], bf16x8 (&kf)[2][NCW]) {
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+      const int key = kv0 + ks * 16 + l16;
+      const bool ok = pg[ks] >= 0;
+      const short* cr =
+          ok ? cache + ((long)pg[ks] * PS + key % PS) * Rp + col0 + lg * 8
+             : cache;
+#pragma unroll
+      for (int dc = 0; dc < NCW; ++dc)
+        kf[ks][dc] = ok ? *reinterpret_cast<const bf16x8*>(cr + dc * 32)
+                        : bf16x8{};
+    }
+  };
+
+  bf16x8 kf[2][NCW];
+  int pg_a[2], pg_b[2];
+  pages_of(kv_lo, pg_a);
+  pages_of(kv_lo + KVT, pg_b);
+  load_tile(kv_lo, pg_a, kf);
+  int buf = 0;
+  short* vt = vt_lds[wid];
+  short* pw = p_lds[wid];
+  for (int kv0 = kv_lo; kv0 <= kv_hi; kv0 += KVT) {
+    const bool more = kv0 + KVT <= kv_hi;
+    pages_of(kv0 + 2 * KVT, pg_a);  // pages of the tile after next
+    // ---- partial scores over this wave's columns
+    f32x4 s[2];
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+      s[ks] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int dc = 0; dc < NCW; ++dc) {
+        bf16v8 kb;
+        __builtin_memcpy(&kb, &kf[ks][dc], 16);
+        s[ks] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[dc], kb, s[ks], 0,
+                                                        0, 0);
+      }
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        s_lds[buf][wid][(lg * 4 + r) * S_STRIDE + ks * 16 + l16] = s[ks][r];
+    }
+    // ---- the same registers, transposed, are this wave's V^T tile
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+      for (int dc = 0; dc < NCW; ++dc)
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+          vt[(dc * 32 + lg * 8 + j) * VT_STRIDE + ks * 16 + l16] =
+              kf[ks][dc][j];
+    // the fragments' last reader is done: the next tile's rows stream into
+    // the same registers while this tile's softmax and PV run
+    if (more) load_tile(kv0 + KVT, pg_b, kf);
+    __syncthreads();
+    // ---- full scores, mask, online softmax (identical in all 4 waves)
+    float alpha[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const bool rok = rt * 16 + lg * 4 + r < H;
+#pragma unroll
+      for (int ks = 0; ks < 2; ++ks) {
+        const int idx = (lg * 4 + r) * S_STRIDE + ks * 16 + l16;
+        const float v = s_lds[buf][0][idx] + s_lds[buf][1][idx] +
+                        s_lds[buf][2][idx] + s_lds[buf][3][idx];
+        const int kpos = kv0 + ks * 16 + l16;
+        s[ks][r] = (rok && kpos <= kv_hi) ? v * scale : -FLT_MAX;
+      }
+      float mx = fmaxf(s[0][r], s[1][r]);
+#pragma unroll
+      for (int off = 1; off < 16; off <<= 1)
+        mx = fmaxf(mx, __shfl_xor(mx, off, WAVE));
+      const float mn = fmaxf(m_run[r], mx);
+      alpha[r] = (m_run[r] == -FLT_MAX) ? 0.f : __expf(m_run[r] - mn);
+      m_run[r] = mn;
+      float rowsum = 0.f;
+#pragma unroll
+      for (int ks = 0; ks < 2; ++ks) {
+        const float p = (s[ks][r] == -FLT_MAX) ? 0.f : __expf(s[ks][r] - mn);
+        s[ks][r] = p;
+        rowsum += p;
+      }
+#pragma unroll
+      for (int off = 1; off < 16; off <<= 1)
+        rowsum += __shfl_xor(rowsum, off, WAVE);
+      l_run[r] = l_run[r] * alpha[r] + rowsum;
+    }
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        pw[(lg * 4 + r) * P_STRIDE + ks * 16 + l16] = f2bits(s[ks][r]);
+    __builtin_amdgcn_s_waitcnt(0xc07f);  // LDS only; global loads stay out
+    const bf16v8 pf =
+        *reinterpret_cast<const bf16v8*>(pw + l16 * P_STRIDE + lg * 8);
+#pragma unroll
+    for (int dt = 0; dt < NDT; ++dt) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) o[dt][r] *= alpha[r];
+      const bf16v8 vf = *reinterpret_cast<const bf16v8*>(
+          vt + (dt * 16 + l16) * VT_STRIDE + lg * 8);
+      o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf, vf, o[dt], 0, 0, 0);
+    }
+    // own-wave WAR on vt / pw: reads above retire before the next writes
+    __builtin_amdgcn_s_waitcnt(0xc07f);
+    pg_b[0] = pg_a[0];
+    pg_b[1] = pg_a[1];
+    buf ^= 1;
+  }
+  // ---- unnormalized partials for this slice
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const int rr = rt * 16 + lg * 4 + r;
+    if (rr >= H) continue;
+    const long pr = ((long)b * n_splits + split) * H + rr;
+    if (wid == 0 && l16 == 0) {
+      part_ml[pr * 2] = m_run[r];
+      part_ml[pr * 2 + 1] = l_run[r];
+    }
+#pragma unroll
+    for (int dt = 0; dt < NDT; ++dt)
+      part_o[pr * Rp + col0 + dt * 16 + l16] = o[dt][r];
+  }
+}
+
 // merge the split-KV partials of one (sequence, head): log-sum-exp rescale
-__global__ __launch_bounds__(64) void latent_attn_combine_kernel(
+__global__ __launch_bounds__(128) void latent_attn_combine_kernel(
     short* __restrict__ out, long o_hs, long o_ts,
     const float* __restrict__ part_o, const float* __restrict__ part_ml,
     const int* __restrict__ seq_lens, int H, int Rp, int n_splits) {
   const int h = blockIdx.x, b = blockIdx.y;
   short* op = out + h * o_hs + (long)b * o_ts;
   if (seq_lens[b] <= 0) {
-    for (int d = threadIdx.x; d < Rp; d += WAVE) op[d] = 0;
+    for (int d = threadIdx.x; d < Rp; d += 128) op[d] = 0;
     return;
   }
   float M = -FLT_MAX;
@@ -431,14 +631,24 @@ __global__ __launch_bounds__(64) void latent_attn_combine_kernel(
     if (m != -FLT_MAX) L += part_ml[pr * 2 + 1] * __expf(m - M);
   }
   const float inv = L > 0.f ? 1.0f / L : 0.f;
-  for (int d = threadIdx.x; d < Rp; d += WAVE) {
-    float acc = 0.f;
+  // Rp is a multiple of 32: 4 consecutive columns per thread
+  for (int d = threadIdx.x * 4; d < Rp; d += 128 * 4) {
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
     for (int s = 0; s < n_splits; ++s) {
       const long pr = ((long)b * n_splits + s) * H + h;
       const float m = part_ml[pr * 2];
-      if (m != -FLT_MAX) acc += part_o[pr * Rp + d] * __expf(m - M);
+      if (m == -FLT_MAX) continue;
+      const float w = __expf(m - M);
+      const float4 v = *reinterpret_cast<const float4*>(part_o + pr * Rp + d);
+      acc[0] = fmaf(v.x, w, acc[0]);
+      acc[1] = fmaf(v.y, w, acc[1]);
+      acc[2] = fmaf(v.z, w, acc[2]);
+      acc[3] = fmaf(v.w, w, acc[3]);
     }
-    op[d] = f2bits(acc * inv);
+    bf16x4 o4;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) o4[j] = f2bits(acc[j] * inv);
+    *reinterpret_cast<bf16x4*>(op + d) = o4;
   }
 }
 
@@ -516,6 +726,9 @@ void latent_window_attention(torch::Tensor out, torch::Tensor q_lat,
                              c10::optional<torch::Tensor> query_lens,
                              double scale, long window, long max_qlen,
                              bool force_simple, long splits) {
+  // splits < 0: run decode on the tile kernel with -splits slices (A/B)
+  const bool force_tile_decode = splits < 0;
+  if (splits < 0) splits = -splits;
   TORCH_CHECK(q_lat.dim() == 3 && out.dim() == 3 && q_lat.stride(2) == 1 &&
               out.stride(2) == 1);
   TORCH_CHECK(cache.dim() == 3 && cache.is_contiguous());
@@ -551,10 +764,44 @@ void latent_window_attention(torch::Tensor out, torch::Tensor q_lat,
 
   const bool bf16 = cache.scalar_type() == at::kBFloat16;
   const bool aligned = (q_lat.stride(0) % 8 == 0) && (q_lat.stride(1) % 8 == 0) &&
-                       (q_lat.storage_offset() % 8 == 0);
+                       (q_lat.storage_offset() % 8 == 0) &&
+                       (out.stride(0) % 8 == 0) && (out.stride(1) % 8 == 0) &&
+                       (out.storage_offset() % 8 == 0);
   if (bf16 && !force_simple && Rp % 32 == 0 && Rp <= 512 && aligned) {
     const int nc = Rp / 32;
     const size_t lds = mfma_lds_bytes(Rp);
+    if (!query_starts.has_value() && !force_tile_decode &&
+        (Rp == 128 || Rp == 256 || Rp == 512)) {
+      // decode: rank-split kernel, several workgroups per CU
+      const int row_tiles = (H + 15) / 16;
+      const long n_max = std::min<long>(window, (long)max_pages * PS);
+      const long want =
+          (512 + (long)B * row_tiles - 1) / ((long)B * row_tiles);
+      long ns = splits > 0 ? splits : std::min<long>(want, n_max / 64);
+      if (ns < 1) ns = 1;
+      auto fo = torch::TensorOptions().dtype(torch::kFloat).device(out.device());
+      auto part_o = torch::empty({(long)B * ns * H * Rp}, fo);
+      auto part_ml = torch::empty({(long)B * ns * H * 2}, fo);
+      dim3 grid(B, ns, row_tiles);
+#define LD_LAUNCH(NCW)                                                         \
+  hipLaunchKernelGGL(latent_decode_mfma_kernel<NCW>, grid, dim3(256), 0,       \
+                     stream, part_o.data_ptr<float>(),                         \
+                     part_ml.data_ptr<float>(), (const short*)q_lat.data_ptr(),\
+                     (long)q_lat.stride(0), (long)q_lat.stride(1),             \
+                     (const short*)cache.data_ptr(),                           \
+                     page_table.data_ptr<int>(), seq_lens.data_ptr<int>(),     \
+                     (float)scale, (int)window, H, PS, max_pages, (int)ns)
+      if (Rp == 128) LD_LAUNCH(1);
+      else if (Rp == 256) LD_LAUNCH(2);
+      else LD_LAUNCH(4);
+#undef LD_LAUNCH
+      hipLaunchKernelGGL(latent_attn_combine_kernel, dim3(H, B), dim3(128), 0,
+                         stream, (short*)out.data_ptr(), (long)out.stride(0),
+                         (long)out.stride(1), part_o.data_ptr<float>(),
+                         part_ml.data_ptr<float>(), seq_lens.data_ptr<int>(),
+                         H, Rp, (int)ns);
+      return;
+    }
     const long rows = max_qlen * H;
     const int row_blocks = (rows + ROWS_PER_BLOCK - 1) / ROWS_PER_BLOCK;
     // decode: too few (sequence, row-block) pairs to fill 256 CUs — cut
@@ -606,7 +853,7 @@ void latent_window_attention(torch::Tensor out, torch::Tensor q_lat,
     else LA_LAUNCH(16);
 #undef LA_LAUNCH
     if (launched && n_splits > 0)
-      hipLaunchKernelGGL(latent_attn_combine_kernel, dim3(H, B), dim3(64), 0,
+      hipLaunchKernelGGL(latent_attn_combine_kernel, dim3(H, B), dim3(128), 0,
                          stream, (short*)out.data_ptr(), (long)out.stride(0),
                          (long)out.stride(1), part_o.data_ptr<float>(),
                          part_ml.data_ptr<float>(), seq_lens.data_ptr<int>(),
