@@ -271,7 +271,7 @@ def test_greedy_generation_through_scheduler(tmp_path, device):
     # nothing a multiple of 32, rank padded inside the pool
     dict(width=48, heads=3, dim=8, vdim=20, q_rank=24, kv_rank=40, groups=3,
          window=23, ff=56, expert_ff=12, experts=7, top=3),
-    dict(width=72, heads=5, dim=24, vdim=8, q_rank=40, kv_rank=136, groups=1,
+    dict(width=72, heads=5, dim=24, vdim=8, q_rank=40, kv_rank=152, groups=1,
          window=130, ff=40, expert_ff=20, experts=3, top=1)])
 def test_bf16_serving_path_close_to_oracle(tmp_path, shape):
     """bf16 serving precision (MFMA tile attention, captured decode graph):
