@@ -102,6 +102,44 @@ class LatentLayout:
                                                 pool.size(2)))
 
 
+class HeadKVLayout:
+    """Per layer a K pool [P, PS, G_l, D_l] and a V pool [P, PS, G_l, Dv_l]
+    (row = token, then kv head): the head count and the key / value sizes
+    may differ from layer to layer and from each other. Checkpoint images
+    are sized by the widest layer."""
+
+    def __init__(self, shapes):
+        # shapes: per layer (kv_heads, key_dim, value_dim)
+        self.shapes = [tuple(int(v) for v in s) for s in shapes]
+        self.n_layers = len(self.shapes)
+
+    def alloc(self, n_pages, page_size, device, dtype):
+        return [(torch.zeros(n_pages, page_size, g, d, dtype=dtype,
+                             device=device),
+                 torch.zeros(n_pages, page_size, g, dv, dtype=dtype,
+                             device=device))
+                for g, d, dv in self.shapes]
+
+    def page_elems(self, page_size: int) -> int:
+        return max(g * (d + dv) for g, d, dv in self.shapes) * page_size
+
+    def gather(self, entry, staging, page_ids):
+        ids = page_ids.long()
+        nk = entry[0][0].numel()
+        nv = entry[1][0].numel()
+        staging[:, :nk] = entry[0].index_select(0, ids).view(-1, nk)
+        staging[:, nk:nk + nv] = entry[1].index_select(0, ids).view(-1, nv)
+
+    def scatter(self, entry, staging, page_ids):
+        ids = page_ids.long()
+        nk = entry[0][0].numel()
+        nv = entry[1][0].numel()
+        entry[0].index_copy_(0, ids, staging[:, :nk].reshape(
+            -1, *entry[0].shape[1:]))
+        entry[1].index_copy_(0, ids, staging[:, nk:nk + nv].reshape(
+            -1, *entry[1].shape[1:]))
+
+
 class KVCacheManager:
     def __init__(self, n_layers: int, n_kv: int, head_dim: int, page_size: int,
                  n_pages: int, device="cpu", dtype=torch.bfloat16,

@@ -1392,32 +1392,30 @@ class LLMEngine:
 
     def validate_model(self, model: str) -> None:
         from ..models.mixtral import MIXTRAL_CONFIGS
-        from ..models.lelitar import LELITAR_CONFIGS
+        from ..models.registry import named_models
+        families = named_models()
         if (model in LLAMA_CONFIGS or model in MIXTRAL_CONFIGS
-                or model in LELITAR_CONFIGS):
+                or model in families):
             return
         from .echo import ECHO_MODELS
         if model in ECHO_MODELS:
             return
         if os.path.isdir(os.path.expanduser(model)):
             return  # weights directory
-        from ..models.mixtral import MIXTRAL_CONFIGS as _MC
         raise ModelNotFound(
             f"unknown model {model!r}; known: "
-            f"{sorted(LLAMA_CONFIGS) + sorted(_MC) + sorted(LELITAR_CONFIGS)}"
+            f"{sorted(LLAMA_CONFIGS) + sorted(MIXTRAL_CONFIGS) + sorted(families)}"
             " + echo")
 
     def _make_instance(self, model: str) -> ModelInstance:
         from ..models.mixtral import MIXTRAL_CONFIGS, make_mixtral_instance
-        from ..models.lelitar import (LELITAR_CONFIGS, is_lelitar_checkpoint,
-                                      make_lelitar_instance)
-        if model in LELITAR_CONFIGS:
-            return make_lelitar_instance(model, self.device, self.engine_cfg)
-        if os.path.isdir(os.path.expanduser(model)) and is_lelitar_checkpoint(
-                os.path.expanduser(model)):
-            # the checkpoint's config.json names its architecture
-            return make_lelitar_instance(model, self.device, self.engine_cfg,
-                                         weights_path=os.path.expanduser(model))
+        from ..models import registry
+        # a named config of a registered family, or a checkpoint whose
+        # config.json names one as its architecture
+        arch = registry.family_of(model)
+        if arch is not None:
+            return registry.make_instance(arch, model, self.device,
+                                          self.engine_cfg)
         if (self.device.startswith("cuda") and torch.cuda.is_available()
                 and not ops.hip_available()):
             raise RuntimeError(

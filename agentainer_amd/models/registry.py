@@ -1,0 +1,64 @@
+"""Model families that bring their own config reader, model class and HIP
+module, keyed by the "architecture" a checkpoint's config.json names.
+
+The engine asks here before falling back to the Llama / Qwen2 loader, and
+tools that compile on first use ask which build target a model needs.
+"""
+
+from __future__ import annotations
+
+import importlib
+import json
+import os
+from typing import Dict, Optional, Tuple
+
+# architecture -> (module, named-config table, instance factory, build target)
+FAMILIES: Dict[str, Tuple[str, str, str, str]] = {
+    "Lelitar": ("agentainer_amd.models.lelitar", "LELITAR_CONFIGS",
+                "make_lelitar_instance", "latent"),
+    "Volalorn": ("agentainer_amd.models.volalorn", "VOLALORN_CONFIGS",
+                 "make_volalorn_instance", "masked"),
+}
+
+
+def checkpoint_architecture(path: str) -> Optional[str]:
+    """The "architecture" string of a checkpoint directory's config.json,
+    or None when there is no such file or key."""
+    try:
+        with open(os.path.join(os.path.expanduser(path), "config.json")) as f:
+            arch = json.load(f).get("architecture")
+    except (OSError, ValueError):
+        return None
+    return arch if isinstance(arch, str) else None
+
+
+def named_models() -> Dict[str, str]:
+    """name -> architecture of every named random-init config."""
+    out = {}
+    for arch, (mod, table, _f, _t) in FAMILIES.items():
+        for name in getattr(importlib.import_module(mod), table):
+            out[name] = arch
+    return out
+
+
+def family_of(model: str) -> Optional[str]:
+    """Architecture of a named config or checkpoint directory, if one of
+    the registered families serves it."""
+    arch = named_models().get(model)
+    if arch is None and os.path.isdir(os.path.expanduser(model)):
+        arch = checkpoint_architecture(model)
+    return arch if arch in FAMILIES else None
+
+
+def make_instance(arch: str, model: str, device: str, engine_cfg):
+    mod, _table, factory, _t = FAMILIES[arch]
+    path = os.path.expanduser(model)
+    return getattr(importlib.import_module(mod), factory)(
+        model, device, engine_cfg,
+        weights_path=path if os.path.isdir(path) else None)
+
+
+def build_target(model: str) -> str:
+    """ops.build target holding the kernels `model` runs on."""
+    arch = family_of(model)
+    return FAMILIES[arch][3] if arch else "core"

@@ -219,8 +219,10 @@ def _skinny_ws(device, N: int, split: int) -> torch.Tensor:
 
 
 def linear(x: torch.Tensor, w: torch.Tensor,
-           w_packed: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """x[M,K] @ w[N,K]^T. Decode-shaped (M<=64) GPU GEMMs go to the
+           w_packed: Optional[torch.Tensor] = None,
+           bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """x[M,K] @ w[N,K]^T (+ bias, added in the library GEMM's epilogue).
+    Decode-shaped (M<=64) GPU GEMMs go to the
     hand-written skinny MFMA kernel — packed-weight variant when the
     caller pre-packed W (streams at the HBM roofline); everything else to
     hipBLASLt via F.linear."""
@@ -230,7 +232,7 @@ def linear(x: torch.Tensor, w: torch.Tensor,
     if (x.is_cuda and M <= 64 and N % 64 == 0 and K % 256 == 0
             and x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16
             and (tuned is not None or SKINNY_FORCED) and not SKINNY_DISABLED
-            and hip_available()):
+            and bias is None and hip_available()):
         mod = _dispatch("skinny_gemm", x)
         split, kc = tuned if tuned else (_skinny_split(N // 64, K), 128)
         if SKINNY_KC:
@@ -245,7 +247,7 @@ def linear(x: torch.Tensor, w: torch.Tensor,
         else:
             mod.skinny_gemm(out, x.contiguous(), w, ws, split)
         return out
-    return torch.nn.functional.linear(x, w)
+    return torch.nn.functional.linear(x, w, bias)
 
 
 def quantize_weight_fp8(w: torch.Tensor):
@@ -520,4 +522,126 @@ def routed_scaled_silu_mul(out, gu, weight):
         mod.routed_scaled_silu_mul(out, gu, weight)
     else:
         reference.routed_scaled_silu_mul(out, gu, weight)
+    return out
+
+
+# ---------------------------------------------------------------------
+# Scalar-gain post-norm, PolyNorm, partial rotary (+YaRN) with q/k norms,
+# masked attention (chunk / window masks; softmax or sigmoid weights) over
+# per-head K/V pools. Own extension (_hip_masked.so), same policy: required
+# on a GPU, fp32 torch references on CPU.
+# ---------------------------------------------------------------------
+
+_masked = None
+_masked_err: Optional[str] = None
+
+
+def _load_masked():
+    global _masked, _masked_err
+    if _masked is not None or _masked_err is not None:
+        return _masked
+    so = os.path.join(os.path.dirname(__file__), "_hip_masked.so")
+    if not os.path.exists(so):
+        _masked_err = (f"HIP extension not built ({so} missing); run "
+                       "python -m agentainer_amd.ops.build masked")
+        return None
+    try:
+        import importlib.util
+
+        spec = importlib.util.spec_from_file_location(
+            "agentainer_amd.ops._hip_masked", so)
+        mod = importlib.util.module_from_spec(spec)
+        spec.loader.exec_module(mod)
+        _masked = mod
+    except Exception as exc:  # noqa: BLE001
+        _masked_err = f"HIP extension failed to load: {exc}"
+    return _masked
+
+
+def masked_available() -> bool:
+    return _load_masked() is not None
+
+
+def _dispatch_masked(name: str, t: torch.Tensor):
+    if t.is_cuda:
+        mod = _load_masked()
+        if mod is None:
+            raise RuntimeError(
+                f"op {name!r} on GPU requires the gfx950 HIP extension: "
+                f"{_masked_err}")
+        return mod
+    return None
+
+
+MASK_CAUSAL = reference.MASK_CAUSAL
+MASK_WINDOW = reference.MASK_WINDOW
+MASK_CHUNK = reference.MASK_CHUNK
+rotary_frequencies = reference.rotary_frequencies
+
+
+def scalar_postnorm_residual(x_res, y, gain, eps: float, h_out):
+    """x_res(fp32) += gain * y / rms(y); h_out = x_res in the compute dtype."""
+    mod = _dispatch_masked("scalar_postnorm_residual", x_res)
+    if mod:
+        mod.scalar_postnorm_residual(x_res, y, gain, float(eps), h_out)
+    else:
+        reference.scalar_postnorm_residual(x_res, y, gain, eps, h_out)
+    return h_out
+
+
+def scalar_rmsnorm(out, x, gain, eps: float):
+    mod = _dispatch_masked("scalar_rmsnorm", x)
+    if mod:
+        mod.scalar_rmsnorm(out, x, gain, float(eps))
+    else:
+        reference.scalar_rmsnorm(out, x, gain, eps)
+    return out
+
+
+def poly_norm(out, z, coef, eps: float):
+    mod = _dispatch_masked("poly_norm", z)
+    if mod:
+        mod.poly_norm(out, z, coef, float(eps))
+    else:
+        reference.poly_norm(out, z, coef, eps)
+    return out
+
+
+def rotary_norm_append(q, k, v, k_cache, v_cache, freqs, amp: float,
+                       positions, slot_mapping, eps: float, q_w=None,
+                       k_w=None, norm_first: bool = False):
+    mod = _dispatch_masked("rotary_norm_append", q)
+    if mod:
+        mod.rotary_norm_append(q, k, v, k_cache, v_cache, freqs, float(amp),
+                               positions, slot_mapping, float(eps), q_w, k_w,
+                               bool(norm_first))
+    else:
+        reference.rotary_norm_append(q, k, v, k_cache, v_cache, freqs, amp,
+                                     positions, slot_mapping, eps, q_w, k_w,
+                                     norm_first)
+
+
+# AGENTAINER_MASKED_SIMPLE=1 forces the one-wave-per-row kernel (A/B and
+# numerics cross-checks against the MFMA tile kernel)
+MASKED_SIMPLE = os.environ.get("AGENTAINER_MASKED_SIMPLE", "0") == "1"
+
+
+def masked_attention(out, q, k_cache, v_cache, page_table, seq_lens,
+                     query_starts, query_lens, scale: float, mask_kind: int,
+                     mask_size: int, keep_first: int = 0,
+                     sigmoid_weights: bool = False, softcap: float = 0.0,
+                     key_bias=None, head_gate=None, max_qlen: int = 1):
+    mod = _dispatch_masked("masked_attention", q)
+    if mod:
+        mod.masked_attention(out, q, k_cache, v_cache, page_table, seq_lens,
+                             query_starts, query_lens, float(scale),
+                             int(mask_kind), int(mask_size), int(keep_first),
+                             bool(sigmoid_weights), float(softcap), key_bias,
+                             head_gate, int(max_qlen), bool(MASKED_SIMPLE))
+    else:
+        reference.masked_attention(out, q, k_cache, v_cache, page_table,
+                                   seq_lens, query_starts, query_lens, scale,
+                                   mask_kind, mask_size, keep_first,
+                                   sigmoid_weights, softcap, key_bias,
+                                   head_gate)
     return out

@@ -12,6 +12,8 @@ paged-cache layouts k_cache [P, n_kv, D/8, PS, 8] / v_cache [P, n_kv, PS, D].
 
 from __future__ import annotations
 
+import math
+
 
 import torch
 
@@ -311,3 +313,183 @@ def routed_scaled_silu_mul(out: torch.Tensor, gu: torch.Tensor,
     g = g3[..., :F_] * w
     u = g3[..., F_:] * w
     out.copy_((g * torch.sigmoid(g) * u).view(T, E * F_).to(out.dtype))
+
+
+# ---------------------------------------------------------------------
+# Scalar-gain norms, PolyNorm, partial rotary (+YaRN) with q/k norms, and
+# masked attention (chunk / window-with-kept-prefix masks, softmax or
+# per-key sigmoid weights) over per-head paged K/V pools.
+# ---------------------------------------------------------------------
+
+def _unit(v: torch.Tensor, eps: float) -> torch.Tensor:
+    return v * torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + eps)
+
+
+def scalar_postnorm_residual(x_res: torch.Tensor, y: torch.Tensor,
+                             gain: torch.Tensor, eps: float,
+                             h_out: torch.Tensor) -> None:
+    """Post-norm residual step: x_res (fp32, in place) += gain * y/rms(y)
+    with ONE gain for the whole row; h_out receives the updated stream in
+    the compute dtype (the next sublayer's GEMM input)."""
+    x_res.add_(_unit(y.float(), eps) * gain.float().reshape(()))
+    h_out.copy_(x_res.to(h_out.dtype))
+
+
+def scalar_rmsnorm(out: torch.Tensor, x: torch.Tensor, gain: torch.Tensor,
+                   eps: float) -> None:
+    out.copy_((_unit(x.float(), eps) * gain.float().reshape(())
+               ).to(out.dtype))
+
+
+def poly_norm(out: torch.Tensor, z: torch.Tensor, coef: torch.Tensor,
+              eps: float) -> None:
+    """out = a U(z) + b U(z^2) + c U(z^3) + e, U = unit rms over the row,
+    powers elementwise, coef = (a, b, c, e) fp32."""
+    zf = z.float()
+    c = coef.float()
+    z2 = zf * zf
+    out.copy_((c[0] * _unit(zf, eps) + c[1] * _unit(z2, eps)
+               + c[2] * _unit(z2 * zf, eps) + c[3]).to(out.dtype))
+
+
+def rotary_frequencies(dims: int, base: float, scaling=None, device="cpu"):
+    """(freqs fp32 [dims/2], amplitude) of a rotary embedding over `dims`
+    coordinates: f_i = base^(-2i/dims). `scaling` = dict(factor, original,
+    fast, slow) applies YaRN: with d(t) = dims ln(original / (2 pi t)) /
+    (2 ln base), lo = max(floor(d(fast)), 0), hi = min(ceil(d(slow)),
+    dims-1) and ramp_i = clamp((i-lo)/max(hi-lo, .001), 0, 1), the
+    frequency becomes f_i/factor * ramp_i + f_i (1-ramp_i) and cos/sin are
+    scaled by 0.1 ln(factor) + 1. Computed in double, stored fp32."""
+    half = dims // 2
+    i = torch.arange(half, dtype=torch.float64)
+    f = torch.pow(torch.tensor(float(base), dtype=torch.float64),
+                  -2.0 * i / dims)
+    amp = 1.0
+    if scaling:
+        factor = float(scaling["factor"])
+        orig = float(scaling["original"])
+
+        def corr(turns):
+            return (dims * math.log(orig / (2 * math.pi * turns))
+                    / (2 * math.log(base)))
+
+        lo = max(math.floor(corr(float(scaling["fast"]))), 0)
+        hi = min(math.ceil(corr(float(scaling["slow"]))), dims - 1)
+        ramp = ((i - lo) / max(hi - lo, 0.001)).clamp(0.0, 1.0)
+        f = f / factor * ramp + f * (1.0 - ramp)
+        amp = 0.1 * math.log(factor) + 1.0
+    return f.to(torch.float32).to(device), float(amp)
+
+
+def _rotate_half(u: torch.Tensor, positions: torch.Tensor,
+                 freqs: torch.Tensor, amp: float) -> torch.Tensor:
+    """u fp32 [T, heads, D]; the first 2*len(freqs) coordinates of every
+    head rotate, coordinate i paired with i + len(freqs)."""
+    half = freqs.numel()
+    ang = positions.to(torch.float32).unsqueeze(1) * freqs.unsqueeze(0)
+    c = (torch.cos(ang) * amp).unsqueeze(1)
+    s = (torch.sin(ang) * amp).unsqueeze(1)
+    a, b = u[..., :half], u[..., half:2 * half]
+    return torch.cat([a * c - b * s, b * c + a * s, u[..., 2 * half:]], -1)
+
+
+def rotary_norm_append(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
+                       k_cache: torch.Tensor, v_cache: torch.Tensor,
+                       freqs: torch.Tensor, amp: float,
+                       positions: torch.Tensor, slot_mapping: torch.Tensor,
+                       eps: float, q_w=None, k_w=None,
+                       norm_first: bool = False) -> None:
+    """Prepare one step's queries and keys and append K/V to the pools.
+
+    q [T, H, D] (rewritten in place), k [T, G, D], v [T, G, Dv]; pools
+    k_cache [P, PS, G, D], v_cache [P, PS, G, Dv]; slot = page*PS + offset
+    (slot < 0 skips the append). Per head, in fp32:
+      norm_first: u <- rms_norm(u) * w, then rotate   (w = q_w / k_w [D])
+      otherwise : u <- rotate(u), then unit rms (no weight)."""
+    def prep(u, w):
+        u = u.float()
+        if norm_first:
+            u = _unit(u, eps)
+            if w is not None:
+                u = u * w.float()
+            return _rotate_half(u, positions, freqs, amp)
+        return _unit(_rotate_half(u, positions, freqs, amp), eps)
+
+    q.copy_(prep(q, q_w).to(q.dtype))
+    kk = prep(k, k_w).to(k_cache.dtype)
+    G, D, Dv = k.size(1), k.size(2), v.size(2)
+    ok = slot_mapping >= 0
+    rows = slot_mapping[ok].long()
+    k_cache.view(-1, G, D)[rows] = kk[ok]
+    v_cache.view(-1, G, Dv)[rows] = v[ok].to(v_cache.dtype)
+
+
+MASK_CAUSAL, MASK_WINDOW, MASK_CHUNK = 0, 1, 2
+
+
+def mask_visible(qpos: torch.Tensor, kpos: torch.Tensor, kind: int,
+                 size: int, keep_first: int) -> torch.Tensor:
+    """Boolean visibility of key positions for query positions.
+    causal: j <= p.  window: j <= p and (p - j < size or j < keep_first).
+    chunk: j <= p and floor(p/size) == floor(j/size)."""
+    seen = kpos <= qpos
+    if kind == MASK_WINDOW:
+        seen = seen & ((qpos - kpos < size) | (kpos < keep_first))
+    elif kind == MASK_CHUNK:
+        seen = seen & (torch.div(qpos, size, rounding_mode="floor")
+                       == torch.div(kpos, size, rounding_mode="floor"))
+    return seen
+
+
+def masked_attention(out: torch.Tensor, q: torch.Tensor,
+                     k_cache: torch.Tensor, v_cache: torch.Tensor,
+                     page_table: torch.Tensor, seq_lens: torch.Tensor,
+                     query_starts, query_lens, scale: float, mask_kind: int,
+                     mask_size: int, keep_first: int, sigmoid_weights: bool,
+                     softcap: float, key_bias, head_gate) -> None:
+    """Grouped-query attention over paged per-head K/V pools.
+
+    out [T, H, Dv], q [T, H, D]; query head h reads kv head h // (H/G).
+    score = <q, k> * scale, then softcap * tanh(score / softcap) when
+    softcap > 0. Weights are a softmax over the visible keys, or (with
+    sigmoid_weights) sigmoid(score + key_bias[h]) per visible key without
+    normalization. head_gate [T, H], when given, multiplies head h's
+    output by sigmoid(head_gate[t, h]). query_starts/query_lens None means
+    one new token per sequence; rows with seq_len <= 0 come back zero."""
+    H = q.size(1)
+    PS, G, D = k_cache.size(1), k_cache.size(2), k_cache.size(3)
+    Dv = v_cache.size(3)
+    kf = k_cache.view(-1, G, D)
+    vf = v_cache.view(-1, G, Dv)
+    rep = H // G
+    B = seq_lens.numel()
+    for b in range(B):
+        total = int(seq_lens[b])
+        qlen = 1 if query_lens is None else int(query_lens[b])
+        start = b if query_starts is None else int(query_starts[b])
+        if total <= 0 or qlen == 0:
+            if total <= 0 and query_lens is None:
+                out[start] = 0
+            continue
+        pos = torch.arange(total)
+        rows = (page_table[b, (pos // PS).long()].long() * PS + pos % PS)
+        K = kf[rows].float().repeat_interleave(rep, dim=1)    # [n, H, D]
+        V = vf[rows].float().repeat_interleave(rep, dim=1)
+        Q = q[start:start + qlen].float()
+        s = torch.einsum("qhd,nhd->hqn", Q, K) * scale
+        if softcap > 0:
+            s = softcap * torch.tanh(s / softcap)
+        qpos = (total - qlen + torch.arange(qlen)).view(1, qlen, 1)
+        seen = mask_visible(qpos, pos.view(1, 1, -1), mask_kind, mask_size,
+                            keep_first)
+        if sigmoid_weights:
+            if key_bias is not None:
+                s = s + key_bias.float().view(H, 1, 1)
+            p = torch.sigmoid(s) * seen
+        else:
+            p = torch.softmax(s.masked_fill(~seen, float("-inf")), dim=-1)
+        o = torch.einsum("hqn,nhe->qhe", p, V)
+        if head_gate is not None:
+            o = o * torch.sigmoid(head_gate[start:start + qlen].float()
+                                  ).unsqueeze(-1)
+        out[start:start + qlen] = o.to(out.dtype)
