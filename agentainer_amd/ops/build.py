@@ -40,6 +40,14 @@ LATENT_SOURCES = [
     "routed_ffn.hip",
 ]
 
+# scalar-gain norms, PolyNorm, rotary + q/k norm + append, masked attention
+MASKED_SOURCES = [
+    "masked_bindings.cpp",
+    "scalar_norm.hip",
+    "rotary_norm.hip",
+    "masked_attn.hip",
+]
+
 SOURCES = [
     "bindings.cpp",
     "rmsnorm.hip",
@@ -64,6 +72,11 @@ def _target(target: str):
         return (os.path.join(HERE, f"_hip_latent{sfx}.so"),
                 os.path.join(HERE, "_build_latent" + sfx), LATENT_SOURCES,
                 "_hip_latent")
+    if target == "masked":
+        sfx = "_asan" if ASAN else ""
+        return (os.path.join(HERE, f"_hip_masked{sfx}.so"),
+                os.path.join(HERE, "_build_masked" + sfx), MASKED_SOURCES,
+                "_hip_masked")
     if target != "core":
         raise ValueError(f"unknown build target {target!r}")
     return OUT, OBJ_DIR, SOURCES, "_hip_ops"
@@ -75,6 +88,7 @@ def needs_build(target: str = "core") -> bool:
         return True
     srcs = [os.path.join(CSRC, s) for s in SOURCES]
     srcs.append(os.path.join(CSRC, "common.h"))
+    srcs.append(os.path.join(CSRC, "latent_common.h"))
     srcs.append(os.path.abspath(__file__))
     return _newest(srcs) > os.path.getmtime(OUT)
 
@@ -83,7 +97,8 @@ def build(verbose: bool = True, force: bool = False,
           target: str = "core") -> str:
     if target == "all":
         build(verbose, force, "core")
-        return build(verbose, force, "latent")
+        build(verbose, force, "latent")
+        return build(verbose, force, "masked")
     OUT, OBJ_DIR, SOURCES, modname = _target(target)
     if not force and not needs_build(target):
         return OUT
@@ -109,7 +124,9 @@ def build(verbose: bool = True, force: bool = False,
         obj = os.path.join(OBJ_DIR, os.path.splitext(src)[0] + ".o")
         objs.append(obj)
         if (os.path.exists(obj)
-                and os.path.getmtime(obj) > _newest([src_path, os.path.join(CSRC, "common.h")])
+                and os.path.getmtime(obj) > _newest(
+                    [src_path, os.path.join(CSRC, "common.h"),
+                     os.path.join(CSRC, "latent_common.h")])
                 and not force):
             continue
         san = (["-fsanitize=address", "-shared-libsan"]

@@ -1,0 +1,160 @@
+// Query/key preparation fused with the paged K/V append (gfx950).
+//
+// For every new token and head, in fp32:
+//
+//   norm_first : u <- u / sqrt(mean(u^2) + eps) * w ;  u <- rotate(u)
+//   otherwise  : u <- rotate(u) ;  u <- u / sqrt(mean(u^2) + eps)
+//
+// rotate() turns the first 2*half coordinates of the head: coordinate i is
+// paired with i + half, angle = position * freq[i] (fp32 product, exact
+// cosf/sinf), and cos/sin are scaled by `amp` (1 unless the frequencies
+// are YaRN-stretched). Coordinates from 2*half on pass through.
+//
+// q [T, H, D] is rewritten in place (a strided view of the fused
+// projection's output); k [T, G, D] goes straight into the pool
+// k_cache[P, PS, G, D] at the token's slot and v [T, G, Dv] is copied into
+// v_cache[P, PS, G, Dv] — rotated keys never travel through HBM twice.
+// slot < 0 skips the append. One wave per (token, head); the head vector
+// sits in a private LDS patch so the pair partner may live in any lane.
+
+#include <torch/extension.h>
+#include <ATen/hip/HIPContext.h>
+#include "latent_common.h"
+
+namespace {
+
+constexpr int RN_WAVES = 4;
+
+__device__ __forceinline__ void wave_lds_sync() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+template <typename T>
+__global__ __launch_bounds__(64 * RN_WAVES) void rotary_norm_append_kernel(
+    T* __restrict__ q, long q_ts, long q_hs, const T* __restrict__ k,
+    long k_ts, long k_hs, const T* __restrict__ v, long v_ts, long v_hs,
+    T* __restrict__ k_cache, T* __restrict__ v_cache,
+    const float* __restrict__ freqs, float amp, int half,
+    const int* __restrict__ positions, const long* __restrict__ slots,
+    float eps, const float* __restrict__ q_w, const float* __restrict__ k_w,
+    int norm_first, int n_tok, int H, int G, int D, int Dv) {
+  extern __shared__ float smem[];
+  const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+  const int per_tok = H + 2 * G;
+  const long item = (long)blockIdx.x * RN_WAVES + wave;
+  if (item >= (long)n_tok * per_tok) return;   // whole wave leaves
+  const int t = (int)(item / per_tok), j = (int)(item % per_tok);
+  const long slot = slots[t];
+  if (j >= H + G) {                            // value head: plain copy
+    if (slot < 0) return;
+    const int g = j - H - G;
+    const T* src = v + (long)t * v_ts + (long)g * v_hs;
+    T* dst = v_cache + (slot * G + g) * Dv;
+    for (int i = lane; i < Dv; i += WAVE) dst[i] = src[i];
+    return;
+  }
+  const bool is_q = j < H;
+  if (!is_q && slot < 0) return;
+  float* s = smem + wave * D;
+  const T* src = is_q ? q + (long)t * q_ts + (long)j * q_hs
+                      : k + (long)t * k_ts + (long)(j - H) * k_hs;
+  const float* w = is_q ? q_w : k_w;
+  float ss = 0.f;
+  for (int i = lane; i < D; i += WAVE) {
+    const float u = ldf(src, i);
+    s[i] = u;
+    ss = fmaf(u, u, ss);
+  }
+  if (norm_first) {
+    const float r = 1.0f / sqrtf(wave_sum(ss) / (float)D + eps);
+    for (int i = lane; i < D; i += WAVE)
+      s[i] = s[i] * r * (w != nullptr ? w[i] : 1.0f);
+  }
+  wave_lds_sync();
+  const float pos = (float)positions[t];
+  for (int i = lane; i < half; i += WAVE) {
+    const float ang = pos * freqs[i];
+    const float c = cosf(ang) * amp, sn = sinf(ang) * amp;
+    const float a = s[i], b = s[i + half];
+    s[i] = a * c - b * sn;
+    s[i + half] = b * c + a * sn;
+  }
+  wave_lds_sync();
+  float r = 1.0f;
+  if (!norm_first) {
+    ss = 0.f;
+    for (int i = lane; i < D; i += WAVE) ss = fmaf(s[i], s[i], ss);
+    r = 1.0f / sqrtf(wave_sum(ss) / (float)D + eps);
+  }
+  T* dst = is_q ? q + (long)t * q_ts + (long)j * q_hs
+                : k_cache + (slot * G + (j - H)) * D;
+  for (int i = lane; i < D; i += WAVE) stf(dst, i, s[i] * r);
+}
+
+}  // namespace
+
+void rotary_norm_append(torch::Tensor q, torch::Tensor k, torch::Tensor v,
+                        torch::Tensor k_cache, torch::Tensor v_cache,
+                        torch::Tensor freqs, double amp,
+                        torch::Tensor positions, torch::Tensor slot_mapping,
+                        double eps, c10::optional<torch::Tensor> q_w,
+                        c10::optional<torch::Tensor> k_w, bool norm_first) {
+  TORCH_CHECK(q.dim() == 3 && k.dim() == 3 && v.dim() == 3 &&
+              q.stride(2) == 1 && k.stride(2) == 1 && v.stride(2) == 1);
+  const int T_ = q.size(0), H = q.size(1), D = q.size(2);
+  const int G = k.size(1), Dv = v.size(2);
+  TORCH_CHECK(k.size(0) == T_ && v.size(0) == T_ && k.size(2) == D &&
+              v.size(1) == G, "q/k/v shapes disagree");
+  TORCH_CHECK(k_cache.dim() == 4 && k_cache.is_contiguous() &&
+              k_cache.size(2) == G && k_cache.size(3) == D,
+              "k_cache must be contiguous [P, PS, G, D]");
+  TORCH_CHECK(v_cache.dim() == 4 && v_cache.is_contiguous() &&
+              v_cache.size(2) == G && v_cache.size(3) == Dv &&
+              v_cache.size(0) == k_cache.size(0) &&
+              v_cache.size(1) == k_cache.size(1),
+              "v_cache must be contiguous [P, PS, G, Dv]");
+  TORCH_CHECK(k.scalar_type() == q.scalar_type() &&
+              v.scalar_type() == q.scalar_type() &&
+              k_cache.scalar_type() == q.scalar_type() &&
+              v_cache.scalar_type() == q.scalar_type(),
+              "q, k, v and the pools share one element type");
+  TORCH_CHECK(freqs.scalar_type() == at::kFloat && freqs.is_contiguous() &&
+              freqs.is_cuda());
+  const int half = freqs.numel();
+  TORCH_CHECK(2 * half <= D, "rotary dims exceed the head size");
+  TORCH_CHECK(positions.scalar_type() == at::kInt && positions.numel() == T_ &&
+              positions.is_contiguous());
+  TORCH_CHECK(slot_mapping.scalar_type() == at::kLong &&
+              slot_mapping.numel() == T_ && slot_mapping.is_contiguous());
+  const float* qw = nullptr;
+  const float* kw = nullptr;
+  if (q_w.has_value()) {
+    TORCH_CHECK(q_w->scalar_type() == at::kFloat && q_w->numel() == D &&
+                q_w->is_contiguous());
+    qw = q_w->data_ptr<float>();
+  }
+  if (k_w.has_value()) {
+    TORCH_CHECK(k_w->scalar_type() == at::kFloat && k_w->numel() == D &&
+                k_w->is_contiguous());
+    kw = k_w->data_ptr<float>();
+  }
+  if (T_ == 0) return;
+  const long items = (long)T_ * (H + 2 * G);
+  const size_t smem = (size_t)RN_WAVES * D * sizeof(float);
+  TORCH_CHECK(smem <= 64 * 1024, "head size too large");
+  auto stream = at::hip::getCurrentHIPStream();
+  LATENT_DISPATCH_T(q, {
+    hipLaunchKernelGGL(
+        rotary_norm_append_kernel<T>,
+        dim3((unsigned)((items + RN_WAVES - 1) / RN_WAVES)),
+        dim3(64 * RN_WAVES), smem, stream, (T*)q.data_ptr(), (long)q.stride(0),
+        (long)q.stride(1), (const T*)k.data_ptr(), (long)k.stride(0),
+        (long)k.stride(1), (const T*)v.data_ptr(), (long)v.stride(0),
+        (long)v.stride(1), (T*)k_cache.data_ptr(), (T*)v_cache.data_ptr(),
+        freqs.data_ptr<float>(), (float)amp, half, positions.data_ptr<int>(),
+        slot_mapping.data_ptr<long>(), (float)eps, qw, kw,
+        norm_first ? 1 : 0, T_, H, G, D, Dv);
+  });
+}

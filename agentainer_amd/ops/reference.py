@@ -352,17 +352,18 @@ def poly_norm(out: torch.Tensor, z: torch.Tensor, coef: torch.Tensor,
                + c[2] * _unit(z2 * zf, eps) + c[3]).to(out.dtype))
 
 
-def rotary_frequencies(dims: int, base: float, scaling=None, device="cpu"):
+def rotary_frequencies(dims: int, base: float, scaling=None, device=None):
     """(freqs fp32 [dims/2], amplitude) of a rotary embedding over `dims`
     coordinates: f_i = base^(-2i/dims). `scaling` = dict(factor, original,
     fast, slow) applies YaRN: with d(t) = dims ln(original / (2 pi t)) /
     (2 ln base), lo = max(floor(d(fast)), 0), hi = min(ceil(d(slow)),
     dims-1) and ramp_i = clamp((i-lo)/max(hi-lo, .001), 0, 1), the
     frequency becomes f_i/factor * ramp_i + f_i (1-ramp_i) and cos/sin are
-    scaled by 0.1 ln(factor) + 1. Computed in double, stored fp32."""
+    scaled by 0.1 ln(factor) + 1. Computed in double on the host, stored
+    fp32 on `device` (default: the current default device)."""
     half = dims // 2
-    i = torch.arange(half, dtype=torch.float64)
-    f = torch.pow(torch.tensor(float(base), dtype=torch.float64),
+    i = torch.arange(half, dtype=torch.float64, device="cpu")
+    f = torch.pow(torch.tensor(float(base), dtype=torch.float64, device="cpu"),
                   -2.0 * i / dims)
     amp = 1.0
     if scaling:
@@ -378,7 +379,10 @@ def rotary_frequencies(dims: int, base: float, scaling=None, device="cpu"):
         ramp = ((i - lo) / max(hi - lo, 0.001)).clamp(0.0, 1.0)
         f = f / factor * ramp + f * (1.0 - ramp)
         amp = 0.1 * math.log(factor) + 1.0
-    return f.to(torch.float32).to(device), float(amp)
+    f = f.to(torch.float32)
+    if device is None:      # follow an enclosing `with torch.device(...)`
+        device = torch.empty(0).device
+    return f.to(device), float(amp)
 
 
 def _rotate_half(u: torch.Tensor, positions: torch.Tensor,

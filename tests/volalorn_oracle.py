@@ -98,6 +98,23 @@ def expand_kv(k: torch.Tensor, heads: int) -> torch.Tensor:
     return k.repeat_interleave(heads // G, dim=1)
 
 
+def attend(q, k, v, seen, scale, softcap=None, sigmoid_bias=None):
+    """q [T, H, D], k [T, G, D], v [T, G, Dv], seen [T, T] -> [T, H, Dv].
+    score = <q, k> scale, optionally soft-capped as cap tanh(score / cap).
+    With sigmoid_bias [H]: weight = sigmoid(score + bias[h]) on every seen
+    key, no normalization. Otherwise: softmax over the seen keys."""
+    H = q.size(1)
+    k, v = expand_kv(k, H), expand_kv(v, H)
+    s = torch.einsum("thd,jhd->htj", q, k) * scale
+    if softcap:
+        s = float(softcap) * torch.tanh(s / float(softcap))
+    if sigmoid_bias is not None:
+        p = torch.sigmoid(s + sigmoid_bias.view(H, 1, 1)) * seen
+    else:
+        p = torch.softmax(s.masked_fill(~seen, float("-inf")), dim=-1)
+    return torch.einsum("htj,jhe->the", p, v)
+
+
 def sigmoid_attention(h, w, mx, eps):
     """Mixer "attention" for one whole sequence h [T, W]."""
     T = h.size(0)
@@ -111,14 +128,9 @@ def sigmoid_attention(h, w, mx, eps):
                         rot.get("scaling")), eps)
     k = unit_rms(rotate(k, pos, int(rot["dims"]), float(rot["base"]),
                         rot.get("scaling")), eps)
-    k, v = expand_kv(k, H), expand_kv(v, H)
-    s = torch.einsum("thd,jhd->htj", q, k) * float(mx["scale"])
-    cap = mx.get("softcap")
-    if cap:
-        s = float(cap) * torch.tanh(s / float(cap))
-    p = torch.sigmoid(s + w["pb"].view(H, 1, 1))
-    p = p * chunk_mask(T, int(mx["mask"]["size"]))
-    a = torch.einsum("htj,jhe->the", p, v)
+    seen = chunk_mask(T, int(mx["mask"]["size"]))
+    a = attend(q, k, v, seen, float(mx["scale"]), softcap=mx.get("softcap"),
+               sigmoid_bias=w["pb"])
     a = a * torch.sigmoid(h @ w["g"].t()).unsqueeze(-1)
     return a.reshape(T, H * Dv) @ w["o"].t()
 
@@ -136,12 +148,9 @@ def softmax_attention(h, w, mx, eps):
     k = unit_rms(k, eps) * w["k.norm"]
     q = rotate(q, pos, int(rot["dims"]), float(rot["base"]), rot.get("scaling"))
     k = rotate(k, pos, int(rot["dims"]), float(rot["base"]), rot.get("scaling"))
-    k, v = expand_kv(k, H), expand_kv(v, H)
-    s = torch.einsum("thd,jhd->htj", q, k) * float(mx["scale"])
     seen = window_keep_mask(T, int(mx["mask"]["size"]),
                             int(mx["mask"].get("keep_first", 0)))
-    p = torch.softmax(s.masked_fill(~seen, float("-inf")), dim=-1)
-    a = torch.einsum("htj,jhe->the", p, v)
+    a = attend(q, k, v, seen, float(mx["scale"]))
     return a.reshape(T, H * Dv) @ w["o"].t()
 
 
