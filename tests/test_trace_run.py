@@ -7,11 +7,13 @@ import subprocess
 import sys
 
 import numpy as np
+import pytest
 import torch
 
 sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
 
 import lelitar_oracle as O  # noqa: E402
+import volalorn_oracle as VO  # noqa: E402
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 TOOL = os.path.join(ROOT, "bin", "trace_run")
@@ -26,9 +28,21 @@ def _run(model, out, steps, dtype="float32", max_tokens=128):
     return p
 
 
-def test_trace_run_mixed_steps_match_oracle(tmp_path):
+def _lelitar_case():
     cfg = O.random_config(vocab=120, window=6, kinds=("moe", "dense", None))
-    w = O.random_weights(cfg, seed=21)
+    return O, cfg, O.random_weights(cfg, seed=21)
+
+
+def _volalorn_case():
+    cfg = VO.make_config(
+        [VO.sigmoid_mixer(chunk=5), VO.softmax_mixer(window=6, keep_first=2),
+         VO.sigmoid_mixer(chunk=16, softcap=None)], vocab=120, no_ff=(1,))
+    return VO, cfg, VO.random_weights(cfg, seed=22)
+
+
+@pytest.mark.parametrize("case", [_lelitar_case, _volalorn_case])
+def test_trace_run_mixed_steps_match_oracle(tmp_path, case):
+    O, cfg, w = case()
     model = str(tmp_path / "ckpt")
     O.save_checkpoint(model, cfg, w)
     g = torch.Generator().manual_seed(3)
