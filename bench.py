@@ -79,10 +79,15 @@ def _parser():
                         "NOT the headline dtype)")
     p.add_argument("--arch-compare", action="store_true",
                    help="instead of the headline workload: prefill and decode "
-                        "tokens/s of the Lelitar design at real-layer sizes "
-                        "beside Llama/Mixtral stacks of equal size")
-    p.add_argument("--arch-sizes", default="s,l,moe",
-                   help="--arch-compare: which size points to run")
+                        "tokens/s of a checkpoint-defined design (see "
+                        "--arch-design) at real-layer sizes beside "
+                        "Llama/Mixtral stacks of equal size")
+    p.add_argument("--arch-sizes", default=None,
+                   help="--arch-compare: which size points to run "
+                        "(default: all points of the design)")
+    p.add_argument("--arch-design", default="lelitar",
+                   choices=["lelitar", "volalorn"],
+                   help="--arch-compare: which design to measure")
     return p
 
 
@@ -130,6 +135,52 @@ def _arch_points():
     return pts
 
 
+def _volalorn_points():
+    """Volalorn size points beside Llama stacks of equal width, head counts
+    and ff: layers alternate the sigmoid/chunk mixer (YaRN rotary on half
+    the head) and the softmax/window mixer (4 kept first tokens). Masks are
+    sized so that a decode step at the benchmark's context reads about as
+    many keys as the Llama stack does."""
+    from agentainer_amd import ops
+    from agentainer_amd.models.llama import LlamaConfig
+    from agentainer_amd.models.volalorn import (MaskedAttentionConfig,
+                                                PolyFeedForwardConfig,
+                                                VolalornConfig,
+                                                VolalornLayerConfig)
+
+    def vol(name, width, heads, kv, chunk, window, ff, n):
+        sig = MaskedAttentionConfig(
+            heads=heads, kv_heads=kv, dim=128, vdim=128, scale=128 ** -0.5,
+            mask_kind=ops.MASK_CHUNK, mask_size=chunk, rot_dims=64,
+            rot_base=500000.0, rot_scaling={"factor": 8.0, "original": 8192,
+                                            "fast": 32.0, "slow": 1.0},
+            softcap=30.0, sigmoid_weights=True, key_bias=True, head_gate=True)
+        soft = MaskedAttentionConfig(
+            heads=heads, kv_heads=kv, dim=128, vdim=128, scale=128 ** -0.5,
+            mask_kind=ops.MASK_WINDOW, mask_size=window, keep_first=4,
+            rot_dims=128, rot_base=500000.0, qkv_bias=True, norm_first=True)
+        layers = [VolalornLayerConfig(
+            "attention" if i % 2 == 0 else "attention_2",
+            sig if i % 2 == 0 else soft, PolyFeedForwardConfig(ff))
+            for i in range(n)]
+        return VolalornConfig(name=name, vocab_size=32000, hidden_size=width,
+                              layers=layers, norm_eps=1e-6, logit_scale=0.5)
+
+    return {
+        "s": ("w2048-ff8192", vol("volalorn-s", 2048, 16, 4, 2048, 1024,
+                                  8192, 4),
+              LlamaConfig(name="llama-s", vocab_size=32000, hidden_size=2048,
+                          n_layers=4, n_heads=16, n_kv_heads=4,
+                          intermediate_size=8192, tie_embeddings=False), None),
+        "l": ("w4096-ff14336", vol("volalorn-l", 4096, 32, 8, 8192, 4096,
+                                   14336, 4),
+              LlamaConfig(name="llama-l", vocab_size=32000, hidden_size=4096,
+                          n_layers=4, n_heads=32, n_kv_heads=8,
+                          intermediate_size=14336, tie_embeddings=False),
+              None),
+    }
+
+
 def run_arch_compare(args):
     """Prefill (8 x 1024-token prompts per step) and decode (64 sequences at
     1024 tokens of context, captured graph) throughput, through the
@@ -137,6 +188,7 @@ def run_arch_compare(args):
     from agentainer_amd.engine.llm import ModelInstance
     from agentainer_amd.models.lelitar import LelitarForCausalLM
     from agentainer_amd.models.mixtral import MixtralForCausalLM
+    from agentainer_amd.models.volalorn import VolalornForCausalLM
 
     dev = "cuda" if torch.cuda.is_available() else "cpu"
     small = dev == "cpu"
@@ -194,18 +246,21 @@ def run_arch_compare(args):
                 "decode_ms": round(dc, 3),
                 "decode_tok_s": round(n_dec / dc * 1e3)}
 
-    pts = _arch_points()
-    for key in args.arch_sizes.split(","):
+    design = args.arch_design
+    pts = _volalorn_points() if design == "volalorn" else _arch_points()
+    ours_cls = (VolalornForCausalLM if design == "volalorn"
+                else LelitarForCausalLM)
+    for key in (args.arch_sizes or ",".join(pts)).split(","):
         label, lcfg, rcfg, kind = pts[key.strip()]
         if small:  # CPU dry run: shrink to something that finishes
             continue
-        ours = measure(lcfg.name, lcfg, LelitarForCausalLM)
+        ours = measure(lcfg.name, lcfg, ours_cls)
         theirs = measure(rcfg.name, rcfg,
                          MixtralForCausalLM if kind == "mixtral" else None)
         print(json.dumps({
             "metric": "arch_compare", "point": label, "layers": rcfg.n_layers,
             "prefill": f"{n_pf}x{pf_len}", "decode": f"{n_dec}@{ctx}",
-            "dtype": "bf16", "data": "synthetic", "lelitar": ours,
+            "dtype": "bf16", "data": "synthetic", design: ours,
             "reference_model": rcfg.name, "reference": theirs,
             "prefill_ratio": round(ours["prefill_tok_s"]
                                    / theirs["prefill_tok_s"], 3),
