@@ -624,6 +624,8 @@ def rotary_norm_append(q, k, v, k_cache, v_cache, freqs, amp: float,
 # AGENTAINER_MASKED_SIMPLE=1 forces the one-wave-per-row kernel (A/B and
 # numerics cross-checks against the MFMA tile kernel)
 MASKED_SIMPLE = os.environ.get("AGENTAINER_MASKED_SIMPLE", "0") == "1"
+# decode key-range slices per (sequence, kv head); 0 = sized to fill the chip
+MASKED_SPLITS = int(os.environ.get("AGENTAINER_MASKED_SPLITS", "0"))
 
 
 def masked_attention(out, q, k_cache, v_cache, page_table, seq_lens,
@@ -637,7 +639,8 @@ def masked_attention(out, q, k_cache, v_cache, page_table, seq_lens,
                              query_starts, query_lens, float(scale),
                              int(mask_kind), int(mask_size), int(keep_first),
                              bool(sigmoid_weights), float(softcap), key_bias,
-                             head_gate, int(max_qlen), bool(MASKED_SIMPLE))
+                             head_gate, int(max_qlen), bool(MASKED_SIMPLE),
+                             int(MASKED_SPLITS))
     else:
         reference.masked_attention(out, q, k_cache, v_cache, page_table,
                                    seq_lens, query_starts, query_lens, scale,

@@ -38,6 +38,7 @@
 
 #include <torch/extension.h>
 #include <ATen/hip/HIPContext.h>
+#include <algorithm>
 #include <cfloat>
 #include "latent_common.h"
 
@@ -423,6 +424,283 @@ __global__ __launch_bounds__(256) void masked_attn_mfma_kernel(
   }
 }
 
+// ------------------------------------------------------------------
+// masked_attn_decode: one new token per sequence, bf16, H/G <= 16
+// ------------------------------------------------------------------
+// A decode step has one query position per sequence: nothing amortizes a
+// block-wide staged tile and barriers would idle three waves of four. Here
+// every WAVE owns whole 32-key tiles: it loads the K fragments of its tile
+// straight from HBM into MFMA A operands, transposes V through a private
+// LDS patch (wave-local synchronization only) and keeps its own (m, l, O)
+// for the group's heads (columns of the MFMA). The visible tiles of the
+// sequence — kept prefix first, then the main range — are dealt round-robin
+// to the 4 waves of n_splits workgroups (grid.x), so a long window spreads
+// over the chip. Waves are merged through LDS; with n_splits > 1 each
+// workgroup writes an un-normalized partial and masked_attn_combine
+// finishes. Latency is hidden by occupancy (several workgroups per CU, each
+// wave with a 32-key tile in flight), not by software pipelining.
+
+__device__ __forceinline__ void wave_lds_sync() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+template <int NDB, int NVB>
+__global__ __launch_bounds__(256) void masked_attn_decode_kernel(
+    short* __restrict__ out, long o_ts, long o_hs, const short* __restrict__ q,
+    long q_ts, long q_hs, const short* __restrict__ kc,
+    const short* __restrict__ vc, const int* __restrict__ page_table,
+    const int* __restrict__ seq_lens, float scale, int kind, int size, int keep,
+    int sigmoid_w, float softcap, const float* __restrict__ key_bias,
+    const short* __restrict__ gate, long g_ts, int H, int G, int nd, int nv,
+    int PS, int max_pages, float* __restrict__ part_o,
+    float* __restrict__ part_ml, int n_splits) {
+  extern __shared__ __attribute__((aligned(16))) short lds[];
+  const int D = nd * 32, Dv = nv * 16;
+  const int split = blockIdx.x, b = blockIdx.y, g = blockIdx.z;
+  const int R = H / G;
+  const int tid = threadIdx.x;
+  const int lane = tid % WAVE, wid = tid / WAVE;
+  const int l16 = lane % 16, lg = lane / 16;
+  const int total = seq_lens[b];
+  const long part_base = ((long)(b * G + g) * n_splits + split) * R;
+
+  if (total <= 0) {  // pad row of a captured batch
+    for (int i = tid; i < R * Dv; i += 256) {
+      const int c = i / Dv, e = i % Dv;
+      if (n_splits == 1) {
+        out[(long)b * o_ts + (long)(g * R + c) * o_hs + e] = 0;
+      } else {
+        part_o[(part_base + c) * Dv + e] = 0.f;
+        if (e == 0) {
+          part_ml[(part_base + c) * 2] = -FLT_MAX;
+          part_ml[(part_base + c) * 2 + 1] = 0.f;
+        }
+      }
+    }
+    return;
+  }
+  const int qpos = total - 1;
+  const int lo = mask_lo(qpos, kind, size);
+  const int* pt = page_table + (long)b * max_pages;
+  const int kt_end = qpos / KVT + 1;
+  const int main_first = lo / KVT;
+  const int n_sink = min((keep + KVT - 1) / KVT, main_first);
+  const int n_vt = n_sink + kt_end - main_first;
+
+  const bool col_ok = l16 < R;
+  const int h = g * R + (col_ok ? l16 : 0);
+  const float bias = (sigmoid_w && key_bias != nullptr) ? key_bias[h] : 0.f;
+  const int cq = col_ok ? qpos : -1;
+
+  bf16v8 qf[NDB];
+  {
+    const short* qp = q + (long)b * q_ts + (long)h * q_hs;
+#pragma unroll
+    for (int c = 0; c < NDB; ++c) {
+      if (c < nd && col_ok)
+        qf[c] = *reinterpret_cast<const bf16v8*>(qp + c * 32 + lg * 8);
+      else
+        qf[c] = bf16v8{};
+    }
+  }
+  f32x4 o[NVB];
+#pragma unroll
+  for (int i = 0; i < NVB; ++i) o[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+  float m = -FLT_MAX, l = 0.f;
+
+  short* vt = lds + (size_t)wid * Dv * VT_STRIDE;   // this wave's V^T patch
+  const int vchunks = Dv / 8;                       // = 2 * nv
+
+  for (int v = split * 4 + wid; v < n_vt; v += 4 * n_splits) {
+    const int kt = v < n_sink ? v : main_first + (v - n_sink);
+    const int t0 = kt * KVT;
+    // K fragments: lane -> key l16 (+16), dims c*32 + lg*8 ..
+    bf16v8 ka[2][NDB];
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb) {
+      const int j = t0 + kb * 16 + l16;
+      const bool ok = j < total;
+      const long row = ok ? (long)pt[j / PS] * PS + j % PS : 0;
+      const short* kr = kc + (row * G + g) * D + lg * 8;
+#pragma unroll
+      for (int c = 0; c < NDB; ++c) {
+        if (c < nd && ok)
+          ka[kb][c] = *reinterpret_cast<const bf16v8*>(kr + c * 32);
+        else
+          ka[kb][c] = bf16v8{};
+      }
+    }
+    // V rows, 16 bytes per lane and load
+    bf16x8 vr[NVB];
+#pragma unroll
+    for (int i = 0; i < NVB; ++i) {
+      vr[i] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
+      if (i < nv) {
+        const int idx = lane + i * WAVE;
+        const int kk = idx / vchunks, ch = idx % vchunks;
+        const int j = t0 + kk;
+        if (j < total) {
+          const long row = (long)pt[j / PS] * PS + j % PS;
+          vr[i] = *reinterpret_cast<const bf16x8*>(
+              vc + (row * G + g) * Dv + ch * 8);
+        }
+      }
+    }
+    wave_lds_sync();   // the previous tile's reads of the patch are done
+#pragma unroll
+    for (int i = 0; i < NVB; ++i) {
+      if (i < nv) {
+        const int idx = lane + i * WAVE;
+        const int kk = idx / vchunks, ch = idx % vchunks;
+        const int slot = vt_slot(kk);
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          vt[(ch * 8 + e) * VT_STRIDE + slot] = vr[i][e];
+      }
+    }
+    wave_lds_sync();
+    f32x4 s0 = f32x4{0.f, 0.f, 0.f, 0.f}, s1 = s0;
+#pragma unroll
+    for (int c = 0; c < NDB; ++c) {
+      if (c < nd) {
+        s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[0][c], qf[c], s0, 0, 0, 0);
+        s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[1][c], qf[c], s1, 0, 0, 0);
+      }
+    }
+    float sv[8], pv[8];
+    bool vis[8];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      sv[r] = s0[r];
+      sv[4 + r] = s1[r];
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const int j = t0 + (e >> 2) * 16 + lg * 4 + (e & 3);
+      vis[e] = j <= cq && (j >= lo || j < keep);
+      float s = sv[e] * scale;
+      if (softcap > 0.f) s = softcap * tanhf(s / softcap);
+      sv[e] = s;
+    }
+    if (sigmoid_w) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e)
+        pv[e] = vis[e] ? sigmoidf_(sv[e] + bias) : 0.f;
+    } else {
+      float tm = -FLT_MAX;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) tm = fmaxf(tm, vis[e] ? sv[e] : -FLT_MAX);
+      tm = fmaxf(tm, __shfl_xor(tm, 16, WAVE));
+      tm = fmaxf(tm, __shfl_xor(tm, 32, WAVE));
+      const float mn = fmaxf(m, tm);
+      const float alpha = (m == -FLT_MAX) ? 0.f : expf(m - mn);
+      float ts = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        pv[e] = vis[e] ? expf(sv[e] - mn) : 0.f;
+        ts += pv[e];
+      }
+      ts += __shfl_xor(ts, 16, WAVE);
+      ts += __shfl_xor(ts, 32, WAVE);
+      l = l * alpha + ts;
+      m = mn;
+#pragma unroll
+      for (int i = 0; i < NVB; ++i)
+        if (i < nv) o[i] *= alpha;
+    }
+    bf16x8 pb;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) pb[e] = f2bits(pv[e]);
+    bf16v8 pf;
+    __builtin_memcpy(&pf, &pb, 16);
+#pragma unroll
+    for (int i = 0; i < NVB; ++i) {
+      if (i < nv) {
+        const bf16v8 af = *reinterpret_cast<const bf16v8*>(
+            vt + (i * 16 + l16) * VT_STRIDE + lg * 8);
+        o[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af, pf, o[i], 0, 0, 0);
+      }
+    }
+  }
+
+  // ---- merge the 4 waves through LDS: fo[wave][e][col], fml[wave][col][2]
+  __syncthreads();
+  float* fo = reinterpret_cast<float*>(lds);
+  float* fml = fo + 4 * Dv * 16;
+#pragma unroll
+  for (int i = 0; i < NVB; ++i) {
+    if (i < nv) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        fo[(wid * Dv + i * 16 + lg * 4 + r) * 16 + l16] = o[i][r];
+    }
+  }
+  if (lg == 0) {
+    fml[(wid * 16 + l16) * 2] = m;
+    fml[(wid * 16 + l16) * 2 + 1] = l;
+  }
+  __syncthreads();
+  for (int i = tid; i < R * Dv; i += 256) {
+    const int c = i / Dv, e = i % Dv;
+    float M = -FLT_MAX;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) M = fmaxf(M, fml[(w * 16 + c) * 2]);
+    float L = 0.f, O = 0.f;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      const float f =
+          sigmoid_w ? 1.0f : expf(fml[(w * 16 + c) * 2] - M);
+      L = fmaf(fml[(w * 16 + c) * 2 + 1], f, L);
+      O = fmaf(fo[(w * Dv + e) * 16 + c], f, O);
+    }
+    if (n_splits == 1) {
+      float mul = sigmoid_w ? 1.0f : 1.0f / L;
+      if (gate != nullptr)
+        mul *= sigmoidf_(bits2f(gate[(long)b * g_ts + g * R + c]));
+      out[(long)b * o_ts + (long)(g * R + c) * o_hs + e] = f2bits(O * mul);
+    } else {
+      part_o[(part_base + c) * Dv + e] = O;
+      if (e == 0) {
+        part_ml[(part_base + c) * 2] = M;
+        part_ml[(part_base + c) * 2 + 1] = L;
+      }
+    }
+  }
+}
+
+// merge the n_splits partials of every (sequence, head): grid (B, H)
+__global__ __launch_bounds__(64) void masked_attn_combine_kernel(
+    short* __restrict__ out, long o_ts, long o_hs,
+    const float* __restrict__ part_o, const float* __restrict__ part_ml,
+    const short* __restrict__ gate, long g_ts, int sigmoid_w, int H, int G,
+    int Dv, int n_splits) {
+  const int b = blockIdx.x, h = blockIdx.y;
+  const int R = H / G, g = h / R, c = h % R;
+  const long base = (long)(b * G + g) * n_splits;
+  float M = -FLT_MAX;
+  for (int s = 0; s < n_splits; ++s)
+    M = fmaxf(M, part_ml[((base + s) * R + c) * 2]);
+  float L = 0.f;
+  for (int s = 0; s < n_splits; ++s) {
+    const float f =
+        sigmoid_w ? 1.0f : expf(part_ml[((base + s) * R + c) * 2] - M);
+    L = fmaf(part_ml[((base + s) * R + c) * 2 + 1], f, L);
+  }
+  float mul = sigmoid_w ? 1.0f : (L > 0.f ? 1.0f / L : 0.f);
+  if (gate != nullptr) mul *= sigmoidf_(bits2f(gate[(long)b * g_ts + h]));
+  for (int e = threadIdx.x; e < Dv; e += WAVE) {
+    float O = 0.f;
+    for (int s = 0; s < n_splits; ++s) {
+      const float f =
+          sigmoid_w ? 1.0f : expf(part_ml[((base + s) * R + c) * 2] - M);
+      O = fmaf(part_o[((base + s) * R + c) * Dv + e], f, O);
+    }
+    out[(long)b * o_ts + (long)h * o_hs + e] = f2bits(O * mul);
+  }
+}
+
 bool aligned16(const void* p) {
   return reinterpret_cast<uintptr_t>(p) % 16 == 0;
 }
@@ -438,7 +716,7 @@ void masked_attention(torch::Tensor out, torch::Tensor q, torch::Tensor k_cache,
                       bool sigmoid_weights, double softcap,
                       c10::optional<torch::Tensor> key_bias,
                       c10::optional<torch::Tensor> head_gate, long max_qlen,
-                      bool force_simple) {
+                      bool force_simple, long splits) {
   TORCH_CHECK(q.dim() == 3 && out.dim() == 3 && q.stride(2) == 1 &&
               out.stride(2) == 1);
   const int T_ = q.size(0), H = q.size(1), D = q.size(2), Dv = out.size(2);
@@ -502,11 +780,58 @@ void masked_attention(torch::Tensor out, torch::Tensor q, torch::Tensor k_cache,
       aligned16(k_cache.data_ptr()) && aligned16(v_cache.data_ptr());
   if (mfma_ok) {
     const int nd = D / 32, nv = Dv / 16;
+    const short* gp =
+        head_gate.has_value() ? (const short*)head_gate->data_ptr() : nullptr;
+    if (!query_starts.has_value() && R <= 16) {
+      // decode: tiles dealt to waves; split long key ranges over workgroups
+      long bound = (long)max_pages * PS;           // keys a query can see
+      if (mask_kind != MK_CAUSAL) bound = std::min(bound, mask_size + keep + 31L);
+      const long tiles = (bound + KVT - 1) / KVT + 1;
+      long n_splits = splits > 0 ? splits : (1024 + (long)B * G - 1) / ((long)B * G);
+      n_splits = std::max(1L, std::min(n_splits, std::max(1L, tiles / 4)));
+      n_splits = std::min(n_splits, 64L);
+      torch::Tensor po, pml;
+      float* pop = nullptr;
+      float* pmlp = nullptr;
+      if (n_splits > 1) {
+        auto opts = torch::TensorOptions().dtype(torch::kFloat).device(q.device());
+        po = torch::empty({(long)B * G * n_splits * R * Dv}, opts);
+        pml = torch::empty({(long)B * G * n_splits * R * 2}, opts);
+        pop = po.data_ptr<float>();
+        pmlp = pml.data_ptr<float>();
+      }
+      const dim3 dgrid((unsigned)n_splits, B, G);
+      const size_t dlds = (size_t)4 * Dv * VT_STRIDE * 2 + 512;
+#define LAUNCH_DECODE(NDB_, NVB_)                                             \
+  hipLaunchKernelGGL((masked_attn_decode_kernel<NDB_, NVB_>), dgrid,          \
+                     dim3(256), dlds, stream, (short*)out.data_ptr(),         \
+                     (long)out.stride(0), (long)out.stride(1),                \
+                     (const short*)q.data_ptr(), (long)q.stride(0),           \
+                     (long)q.stride(1), (const short*)k_cache.data_ptr(),     \
+                     (const short*)v_cache.data_ptr(),                        \
+                     page_table.data_ptr<int>(), seq_lens.data_ptr<int>(),    \
+                     (float)scale, (int)mask_kind, (int)mask_size, keep,      \
+                     sigmoid_weights ? 1 : 0, (float)softcap, kb, gp, g_ts, H, \
+                     G, nd, nv, PS, max_pages, pop, pmlp, (int)n_splits)
+      if (nd <= 4 && nv <= 4) {
+        LAUNCH_DECODE(4, 4);
+      } else if (nd <= 4 && nv <= 8) {
+        LAUNCH_DECODE(4, 8);
+      } else {
+        LAUNCH_DECODE(8, 16);
+      }
+#undef LAUNCH_DECODE
+      if (n_splits > 1) {
+        hipLaunchKernelGGL(masked_attn_combine_kernel, dim3(B, H), dim3(64), 0,
+                           stream, (short*)out.data_ptr(), (long)out.stride(0),
+                           (long)out.stride(1), pop, pmlp, gp, g_ts,
+                           sigmoid_weights ? 1 : 0, H, G, Dv, (int)n_splits);
+      }
+      return;
+    }
     const dim3 grid((unsigned)(((long)max_qlen * R + COLS_PER_BLOCK - 1) /
                                COLS_PER_BLOCK), B, G);
     const size_t lds = ((size_t)KVT * (D + 8) + (size_t)Dv * VT_STRIDE) * 2;
-    const short* gp =
-        head_gate.has_value() ? (const short*)head_gate->data_ptr() : nullptr;
 #define LAUNCH_MFMA(NDB_, NVB_)                                               \
   hipLaunchKernelGGL((masked_attn_mfma_kernel<NDB_, NVB_>), grid, dim3(256),  \
                      lds, stream, (short*)out.data_ptr(),                     \

@@ -23,7 +23,7 @@ void masked_attention(torch::Tensor out, torch::Tensor q, torch::Tensor k_cache,
                       bool sigmoid_weights, double softcap,
                       c10::optional<torch::Tensor> key_bias,
                       c10::optional<torch::Tensor> head_gate, long max_qlen,
-                      bool force_simple);
+                      bool force_simple, long splits);
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.doc() = "agentainer_amd CDNA4 (gfx950) masked-attention family kernels";

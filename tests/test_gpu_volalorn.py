@@ -194,3 +194,40 @@ def test_masked_attention_prompt_and_decode(simple, dtype, H, G, D, Dv, mask):
     torch.testing.assert_close(out_dec[:-1].cpu().float(),
                                out_r[last].float(), **tol)
     assert float(out_dec[-1].abs().max()) == 0.0
+
+
+@pytest.mark.parametrize("splits", [0, 1, 3])
+@pytest.mark.parametrize("mask", [
+    (ref.MASK_WINDOW, 600, 40, False, 0.0, False),
+    (ref.MASK_CHUNK, 512, 0, True, 6.0, True),
+    (ref.MASK_CAUSAL, 0, 0, False, 0.0, True),
+])
+@pytest.mark.parametrize("H,G,D,Dv", [(8, 2, 64, 32), (4, 4, 128, 128),
+                                      (16, 1, 32, 48)])
+def test_masked_attention_long_decode_split(splits, mask, H, G, D, Dv):
+    """Decode over hundreds of keys: the key range is cut into slices whose
+    partial results are merged (softmax statistics, or plain sums for the
+    sigmoid weights)."""
+    kind, size, keep, sig, cap, use_gate = mask
+    lens = [700, 513, 33, 1]
+    qlens = [1, 1, 1, 1]
+    (q, kc, vc, pt, sl, qs, ql, gate, bias) = _attn_case(
+        H + D, H, G, D, Dv, 16, lens, qlens, torch.bfloat16)
+    kw = dict(scale=D ** -0.5 * 2.0, mask_kind=kind, mask_size=size,
+              keep_first=keep, sigmoid_weights=sig, softcap=cap)
+    out_r = torch.zeros(4, H, Dv, dtype=torch.bfloat16)
+    ref.masked_attention(out_r, q, kc, vc, pt, sl, None, None,
+                         key_bias=bias if sig else None,
+                         head_gate=gate if use_gate else None, **kw)
+    prev = ops.MASKED_SPLITS
+    ops.MASKED_SPLITS = splits
+    try:
+        out_d = torch.zeros(4, H, Dv, dtype=torch.bfloat16, device="cuda")
+        ops.masked_attention(out_d, q.cuda(), kc.cuda(), vc.cuda(), pt.cuda(),
+                             sl.cuda(), None, None,
+                             key_bias=bias.cuda() if sig else None,
+                             head_gate=gate.cuda() if use_gate else None, **kw)
+    finally:
+        ops.MASKED_SPLITS = prev
+    tol = dict(rtol=3e-2, atol=3e-2 * (10.0 if sig else 1.0))
+    torch.testing.assert_close(out_d.cpu().float(), out_r.float(), **tol)
