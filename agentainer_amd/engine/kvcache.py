@@ -103,10 +103,11 @@ class LatentLayout:
 
 
 class HeadKVLayout:
-    """Per layer a K pool [P, PS, G_l, D_l] and a V pool [P, PS, G_l, Dv_l]
-    (row = token, then kv head): the head count and the key / value sizes
-    may differ from layer to layer and from each other. Checkpoint images
-    are sized by the widest layer."""
+    """Per layer a K pool [P, G_l, PS, D_l] and a V pool [P, G_l, PS, Dv_l]:
+    inside a page every kv head owns PS consecutive token rows, so the
+    attention kernels stream one contiguous block per (page, head). The
+    head count and the key / value sizes may differ from layer to layer
+    and from each other. Checkpoint images are sized by the widest layer."""
 
     def __init__(self, shapes):
         # shapes: per layer (kv_heads, key_dim, value_dim)
@@ -114,9 +115,9 @@ class HeadKVLayout:
         self.n_layers = len(self.shapes)
 
     def alloc(self, n_pages, page_size, device, dtype):
-        return [(torch.zeros(n_pages, page_size, g, d, dtype=dtype,
+        return [(torch.zeros(n_pages, g, page_size, d, dtype=dtype,
                              device=device),
-                 torch.zeros(n_pages, page_size, g, dv, dtype=dtype,
+                 torch.zeros(n_pages, g, page_size, dv, dtype=dtype,
                              device=device))
                 for g, d, dv in self.shapes]
 

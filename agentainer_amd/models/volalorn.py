@@ -29,7 +29,7 @@ Serving design (what runs on the MI355X):
     kernel (ops.rotary_norm_append) rotates / normalizes q in place and k
     on its way into the paged pool and copies v there. The engine's
     KVCacheManager owns the pools through HeadKVLayout — per layer
-    K [pages, page, G, dim] and V [pages, page, G, vdim].
+    K [pages, G, page, dim] and V [pages, G, page, vdim].
   * ops.masked_attention serves prompt portions and single decoded tokens
     with one kernel family: mask kind / size / kept prefix, soft cap,
     sigmoid-vs-softmax weighting, per-head key bias and the per-head

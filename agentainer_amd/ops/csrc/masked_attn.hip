@@ -1,6 +1,7 @@
 // Masked grouped-query attention over paged per-head K/V pools (gfx950).
 //
-//   k_cache [P, PS, G, D]   v_cache [P, PS, G, Dv]   (row = token, kv head)
+//   k_cache [P, G, PS, D]   v_cache [P, G, PS, Dv]   (a page holds, per kv
+//   head, PS consecutive token rows: one (page, head) block is contiguous)
 //   q [T, H, D], out [T, H, Dv]; query head h reads kv head h / (H/G).
 //
 //   score  = <q, k> * scale;  score <- cap * tanh(score / cap)   (cap > 0)
@@ -109,7 +110,7 @@ __global__ __launch_bounds__(64) void masked_attn_rowwave_kernel(
     float s = -FLT_MAX;
     if (valid) {
       const int j = u < ns ? u : lo + (u - ns);
-      const T* kr = kc + (((long)pt[j / PS] * PS + j % PS) * G + g) * D;
+      const T* kr = kc + ((((long)pt[j / PS] * G + g) * PS) + j % PS) * D;
       float d = 0.f;
       if (vec) {
         for (int i = 0; i < D; i += 4) {
@@ -144,7 +145,7 @@ __global__ __launch_bounds__(64) void masked_attn_rowwave_kernel(
     for (int jj = 0; jj < n; ++jj) {
       const int ug = u0 + jj;
       const int jg = ug < ns ? ug : lo + (ug - ns);
-      const T* vr = vc + (((long)pt[jg / PS] * PS + jg % PS) * G + g) * Dv;
+      const T* vr = vc + ((((long)pt[jg / PS] * G + g) * PS) + jg % PS) * Dv;
       const float pj = p_s[jj];
 #pragma unroll
       for (int k = 0; k < RW_MAX_ACC; ++k) {
@@ -277,9 +278,8 @@ __global__ __launch_bounds__(256) void masked_attn_mfma_kernel(
         const int kk = idx / kchunks, ch = idx % kchunks;
         const int j = t0 + kk;
         if (j < total) {
-          const long row = (long)pt[j / PS] * PS + j % PS;
-          kreg[i] = *reinterpret_cast<const bf16x8*>(
-              kc + (row * G + g) * D + ch * 8);
+          const long row = ((long)pt[j / PS] * G + g) * PS + j % PS;
+          kreg[i] = *reinterpret_cast<const bf16x8*>(kc + row * D + ch * 8);
         }
       }
     }
@@ -291,9 +291,8 @@ __global__ __launch_bounds__(256) void masked_attn_mfma_kernel(
         const int kk = idx / vchunks, ch = idx % vchunks;
         const int j = t0 + kk;
         if (j < total) {
-          const long row = (long)pt[j / PS] * PS + j % PS;
-          vreg[i] = *reinterpret_cast<const bf16x8*>(
-              vc + (row * G + g) * Dv + ch * 8);
+          const long row = ((long)pt[j / PS] * G + g) * PS + j % PS;
+          vreg[i] = *reinterpret_cast<const bf16x8*>(vc + row * Dv + ch * 8);
         }
       }
     }
@@ -522,8 +521,8 @@ __global__ __launch_bounds__(256) void masked_attn_decode_kernel(
     for (int kb = 0; kb < 2; ++kb) {
       const int j = t0 + kb * 16 + l16;
       const bool ok = j < total;
-      const long row = ok ? (long)pt[j / PS] * PS + j % PS : 0;
-      const short* kr = kc + (row * G + g) * D + lg * 8;
+      const long row = ok ? ((long)pt[j / PS] * G + g) * PS + j % PS : 0;
+      const short* kr = kc + row * D + lg * 8;
 #pragma unroll
       for (int c = 0; c < NDB; ++c) {
         if (c < nd && ok)
@@ -542,9 +541,8 @@ __global__ __launch_bounds__(256) void masked_attn_decode_kernel(
         const int kk = idx / vchunks, ch = idx % vchunks;
         const int j = t0 + kk;
         if (j < total) {
-          const long row = (long)pt[j / PS] * PS + j % PS;
-          vr[i] = *reinterpret_cast<const bf16x8*>(
-              vc + (row * G + g) * Dv + ch * 8);
+          const long row = ((long)pt[j / PS] * G + g) * PS + j % PS;
+          vr[i] = *reinterpret_cast<const bf16x8*>(vc + row * Dv + ch * 8);
         }
       }
     }
@@ -723,9 +721,9 @@ void masked_attention(torch::Tensor out, torch::Tensor q, torch::Tensor k_cache,
   TORCH_CHECK(out.size(0) == T_ && out.size(1) == H);
   TORCH_CHECK(k_cache.dim() == 4 && k_cache.is_contiguous() &&
               v_cache.dim() == 4 && v_cache.is_contiguous());
-  const int PS = k_cache.size(1), G = k_cache.size(2);
+  const int G = k_cache.size(1), PS = k_cache.size(2);
   TORCH_CHECK(k_cache.size(3) == D && v_cache.size(3) == Dv &&
-              v_cache.size(2) == G && v_cache.size(1) == PS &&
+              v_cache.size(1) == G && v_cache.size(2) == PS &&
               v_cache.size(0) == k_cache.size(0), "pool shapes disagree");
   TORCH_CHECK(G >= 1 && H % G == 0, "heads % kv_heads != 0");
   TORCH_CHECK(q.scalar_type() == out.scalar_type() &&

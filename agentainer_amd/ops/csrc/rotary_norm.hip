@@ -12,8 +12,8 @@
 //
 // q [T, H, D] is rewritten in place (a strided view of the fused
 // projection's output); k [T, G, D] goes straight into the pool
-// k_cache[P, PS, G, D] at the token's slot and v [T, G, Dv] is copied into
-// v_cache[P, PS, G, Dv] — rotated keys never travel through HBM twice.
+// k_cache[P, G, PS, D] at the token's slot and v [T, G, Dv] is copied into
+// v_cache[P, G, PS, Dv] — rotated keys never travel through HBM twice.
 // slot < 0 skips the append. One wave per (token, head); the head vector
 // sits in a private LDS patch so the pair partner may live in any lane.
 
@@ -39,7 +39,7 @@ __global__ __launch_bounds__(64 * RN_WAVES) void rotary_norm_append_kernel(
     const float* __restrict__ freqs, float amp, int half,
     const int* __restrict__ positions, const long* __restrict__ slots,
     float eps, const float* __restrict__ q_w, const float* __restrict__ k_w,
-    int norm_first, int n_tok, int H, int G, int D, int Dv) {
+    int norm_first, int n_tok, int H, int G, int D, int Dv, int PS) {
   extern __shared__ float smem[];
   const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
   const int per_tok = H + 2 * G;
@@ -51,7 +51,7 @@ __global__ __launch_bounds__(64 * RN_WAVES) void rotary_norm_append_kernel(
     if (slot < 0) return;
     const int g = j - H - G;
     const T* src = v + (long)t * v_ts + (long)g * v_hs;
-    T* dst = v_cache + (slot * G + g) * Dv;
+    T* dst = v_cache + (((slot / PS) * G + g) * PS + slot % PS) * Dv;
     for (int i = lane; i < Dv; i += WAVE) dst[i] = src[i];
     return;
   }
@@ -89,7 +89,7 @@ __global__ __launch_bounds__(64 * RN_WAVES) void rotary_norm_append_kernel(
     r = 1.0f / sqrtf(wave_sum(ss) / (float)D + eps);
   }
   T* dst = is_q ? q + (long)t * q_ts + (long)j * q_hs
-                : k_cache + (slot * G + (j - H)) * D;
+                : k_cache + (((slot / PS) * G + (j - H)) * PS + slot % PS) * D;
   for (int i = lane; i < D; i += WAVE) stf(dst, i, s[i] * r);
 }
 
@@ -108,13 +108,13 @@ void rotary_norm_append(torch::Tensor q, torch::Tensor k, torch::Tensor v,
   TORCH_CHECK(k.size(0) == T_ && v.size(0) == T_ && k.size(2) == D &&
               v.size(1) == G, "q/k/v shapes disagree");
   TORCH_CHECK(k_cache.dim() == 4 && k_cache.is_contiguous() &&
-              k_cache.size(2) == G && k_cache.size(3) == D,
-              "k_cache must be contiguous [P, PS, G, D]");
+              k_cache.size(1) == G && k_cache.size(3) == D,
+              "k_cache must be contiguous [P, G, PS, D]");
   TORCH_CHECK(v_cache.dim() == 4 && v_cache.is_contiguous() &&
-              v_cache.size(2) == G && v_cache.size(3) == Dv &&
+              v_cache.size(1) == G && v_cache.size(3) == Dv &&
               v_cache.size(0) == k_cache.size(0) &&
-              v_cache.size(1) == k_cache.size(1),
-              "v_cache must be contiguous [P, PS, G, Dv]");
+              v_cache.size(2) == k_cache.size(2),
+              "v_cache must be contiguous [P, G, PS, Dv]");
   TORCH_CHECK(k.scalar_type() == q.scalar_type() &&
               v.scalar_type() == q.scalar_type() &&
               k_cache.scalar_type() == q.scalar_type() &&
@@ -155,6 +155,6 @@ void rotary_norm_append(torch::Tensor q, torch::Tensor k, torch::Tensor v,
         (long)v.stride(1), (T*)k_cache.data_ptr(), (T*)v_cache.data_ptr(),
         freqs.data_ptr<float>(), (float)amp, half, positions.data_ptr<int>(),
         slot_mapping.data_ptr<long>(), (float)eps, qw, kw,
-        norm_first ? 1 : 0, T_, H, G, D, Dv);
+        norm_first ? 1 : 0, T_, H, G, D, Dv, (int)k_cache.size(2));
   });
 }

@@ -406,8 +406,9 @@ def rotary_norm_append(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
     """Prepare one step's queries and keys and append K/V to the pools.
 
     q [T, H, D] (rewritten in place), k [T, G, D], v [T, G, Dv]; pools
-    k_cache [P, PS, G, D], v_cache [P, PS, G, Dv]; slot = page*PS + offset
-    (slot < 0 skips the append). Per head, in fp32:
+    k_cache [P, G, PS, D], v_cache [P, G, PS, Dv] (per page and kv head, PS
+    consecutive token rows); slot = page*PS + offset (slot < 0 skips the
+    append). Per head, in fp32:
       norm_first: u <- rms_norm(u) * w, then rotate   (w = q_w / k_w [D])
       otherwise : u <- rotate(u), then unit rms (no weight)."""
     def prep(u, w):
@@ -421,11 +422,12 @@ def rotary_norm_append(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
 
     q.copy_(prep(q, q_w).to(q.dtype))
     kk = prep(k, k_w).to(k_cache.dtype)
-    G, D, Dv = k.size(1), k.size(2), v.size(2)
+    PS = k_cache.size(2)
     ok = slot_mapping >= 0
     rows = slot_mapping[ok].long()
-    k_cache.view(-1, G, D)[rows] = kk[ok]
-    v_cache.view(-1, G, Dv)[rows] = v[ok].to(v_cache.dtype)
+    page, off = rows // PS, rows % PS
+    k_cache[page, :, off] = kk[ok]
+    v_cache[page, :, off] = v[ok].to(v_cache.dtype)
 
 
 MASK_CAUSAL, MASK_WINDOW, MASK_CHUNK = 0, 1, 2
@@ -461,10 +463,7 @@ def masked_attention(out: torch.Tensor, q: torch.Tensor,
     output by sigmoid(head_gate[t, h]). query_starts/query_lens None means
     one new token per sequence; rows with seq_len <= 0 come back zero."""
     H = q.size(1)
-    PS, G, D = k_cache.size(1), k_cache.size(2), k_cache.size(3)
-    Dv = v_cache.size(3)
-    kf = k_cache.view(-1, G, D)
-    vf = v_cache.view(-1, G, Dv)
+    G, PS = k_cache.size(1), k_cache.size(2)
     rep = H // G
     B = seq_lens.numel()
     for b in range(B):
@@ -476,10 +475,10 @@ def masked_attention(out: torch.Tensor, q: torch.Tensor,
                 out[start] = 0
             continue
         pos = torch.arange(total)
-        rows = (page_table[b, (pos // PS).long()].long() * PS + pos % PS)
-        K = kf[rows].float().repeat_interleave(rep, dim=1)    # [n, H, D]
-        V = vf[rows].float().repeat_interleave(rep, dim=1)
-        Q = q[start:start + qlen].float()
+        pages = page_table[b, (pos // PS).long()].long()
+        K = k_cache[pages, :, pos % PS].float().repeat_interleave(rep, dim=1)
+        V = v_cache[pages, :, pos % PS].float().repeat_interleave(rep, dim=1)
+        Q = q[start:start + qlen].float()                     # K [n, H, D]
         s = torch.einsum("qhd,nhd->hqn", Q, K) * scale
         if softcap > 0:
             s = softcap * torch.tanh(s / softcap)

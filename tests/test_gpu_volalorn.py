@@ -87,13 +87,13 @@ def test_rotary_norm_append(dtype, norm_first, H, G, D, Dv, rot):
                 p[:, H * D + G * D:n].view(T, G, Dv))
 
     pr = proj.clone()
-    kc_r = torch.full((P, PS, G, D), 7.0, dtype=dtype)
-    vc_r = torch.full((P, PS, G, Dv), 7.0, dtype=dtype)
+    kc_r = torch.full((P, G, PS, D), 7.0, dtype=dtype)
+    vc_r = torch.full((P, G, PS, Dv), 7.0, dtype=dtype)
     ref.rotary_norm_append(*views(pr), kc_r, vc_r, freqs, amp, pos, slots,
                            1e-5, qw, kw, norm_first)
     pd = proj.cuda()
-    kc_d = torch.full((P, PS, G, D), 7.0, dtype=dtype, device="cuda")
-    vc_d = torch.full((P, PS, G, Dv), 7.0, dtype=dtype, device="cuda")
+    kc_d = torch.full((P, G, PS, D), 7.0, dtype=dtype, device="cuda")
+    vc_d = torch.full((P, G, PS, Dv), 7.0, dtype=dtype, device="cuda")
     ops.rotary_norm_append(*views(pd), kc_d, vc_d, freqs.cuda(), amp,
                            pos.cuda(), slots.cuda(), 1e-5,
                            qw.cuda() if norm_first else None,
@@ -117,8 +117,8 @@ def _attn_case(seed, H, G, D, Dv, PS, lens, qlens, dtype):
     for b, n in enumerate(lens):
         for i in range(-(-n // PS)):
             pt[b, i] = perm.pop()
-    kc = torch.randn(n_pages, PS, G, D, generator=g).to(dtype)
-    vc = torch.randn(n_pages, PS, G, Dv, generator=g).to(dtype)
+    kc = torch.randn(n_pages, G, PS, D, generator=g).to(dtype)
+    vc = torch.randn(n_pages, G, PS, Dv, generator=g).to(dtype)
     T = sum(qlens)
     q = (torch.randn(T, H, D, generator=g) * 1.5).to(dtype)
     gate = torch.randn(T, H, generator=g).to(dtype)

@@ -122,8 +122,8 @@ def test_rotary_norm_append(device, norm_first, H, G, D, Dv, rot):
     freqs, amp = ops.rotary_frequencies(rot, 5000.0, sc)
     qw = torch.rand(D, generator=g) + 0.5
     kw = torch.rand(D, generator=g) + 0.5
-    kc = torch.zeros(P, PS, G, D, device=device)
-    vc = torch.zeros(P, PS, G, Dv, device=device)
+    kc = torch.zeros(P, G, PS, D, device=device)
+    vc = torch.zeros(P, G, PS, Dv, device=device)
     qd = q.clone().to(device)
     ops.rotary_norm_append(qd, k.to(device), v.to(device), kc, vc,
                            freqs.to(device), amp, pos.to(device),
@@ -138,8 +138,9 @@ def test_rotary_norm_append(device, norm_first, H, G, D, Dv, rot):
         k_want = O.unit_rms(O.rotate(k, pos, rot, 5000.0, sc), 1e-4)
     tol = 3e-4  # fp32 cos/sin of angles up to 1000 rad
     close(qd, q_want, tol)
-    close(kc.view(-1, G, D)[slots.to(device)], k_want, tol)
-    close(vc.view(-1, G, Dv)[slots.to(device)], v, 1e-7)
+    sd = slots.to(device)
+    close(kc[sd // PS, :, sd % PS], k_want, tol)
+    close(vc[sd // PS, :, sd % PS], v, 1e-7)
     # coordinates past the rotary dims pass through the rotation untouched
     if not norm_first and rot < D:
         ratio = qd.cpu()[..., rot:] / q[..., rot:]
@@ -154,11 +155,11 @@ def paged(k, v, PS, seed):
     n = -(-T // PS)
     g = torch.Generator().manual_seed(seed)
     order = (torch.randperm(n + 3, generator=g)[:n] + 1).tolist()
-    kc = torch.randn(n + 4, PS, k.size(1), k.size(2), generator=g)
-    vc = torch.randn(n + 4, PS, v.size(1), v.size(2), generator=g)
+    kc = torch.randn(n + 4, k.size(1), PS, k.size(2), generator=g)
+    vc = torch.randn(n + 4, v.size(1), PS, v.size(2), generator=g)
     for t in range(T):
-        kc[order[t // PS], t % PS] = k[t]
-        vc[order[t // PS], t % PS] = v[t]
+        kc[order[t // PS], :, t % PS] = k[t]
+        vc[order[t // PS], :, t % PS] = v[t]
     return kc, vc, torch.tensor([order], dtype=torch.int32)
 
 
@@ -339,8 +340,8 @@ def test_mixer_prompt_then_decode_matches_whole_sequence(device, layer):
     want = O.MIXERS[layer["type"]](h, w, layer["mixer"], eps)
     n_pages = -(-T // PS)
     pages = list(range(n_pages, 0, -1))            # reversed page order
-    kc = torch.zeros(n_pages + 1, PS, mc.kv_heads, mc.dim, device=device)
-    vc = torch.zeros(n_pages + 1, PS, mc.kv_heads, mc.vdim, device=device)
+    kc = torch.zeros(n_pages + 1, mc.kv_heads, PS, mc.dim, device=device)
+    vc = torch.zeros(n_pages + 1, mc.kv_heads, PS, mc.vdim, device=device)
     pt = torch.tensor([pages], dtype=torch.int32, device=device)
 
     def step(lo, hi, prefill):
