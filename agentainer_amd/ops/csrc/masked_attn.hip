@@ -193,7 +193,6 @@ __global__ __launch_bounds__(256) void masked_attn_mfma_kernel(
     int PS, int max_pages) {
   extern __shared__ __attribute__((aligned(16))) short lds[];
   constexpr int KL = NDB / 2;              // 16-byte K loads per thread
-  constexpr int VL = (NVB + 3) / 4;        // 16-byte V loads per thread
   const int D = nd * 32, Dv = nv * 16;
   const int KS = D + 8;                    // padded key row stride
   short* k_lds = lds;                      // [KVT][KS]
@@ -267,7 +266,11 @@ __global__ __launch_bounds__(256) void masked_attn_mfma_kernel(
 
   // ---- staging: global -> registers -> LDS
   const int kchunks = D / 8, vchunks = Dv / 8;     // 16-byte chunks per row
-  bf16x8 kreg[KL], vreg[VL];
+  // V: one unit = 4 consecutive keys x one 8-value chunk, so that the
+  // transposed tile is written 4 keys (8 bytes) at a time; <= 256 units
+  bf16x8 kreg[KL], vreg[4];
+  const bool v_unit = tid < 8 * vchunks;
+  const int v_kq = tid / vchunks, v_ch = tid % vchunks;
   auto load_tile = [&](int kt) {
     const int t0 = kt * KVT;
 #pragma unroll
@@ -284,16 +287,12 @@ __global__ __launch_bounds__(256) void masked_attn_mfma_kernel(
       }
     }
 #pragma unroll
-    for (int i = 0; i < VL; ++i) {
-      const int idx = tid + i * 256;
-      vreg[i] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
-      if (idx < KVT * vchunks) {
-        const int kk = idx / vchunks, ch = idx % vchunks;
-        const int j = t0 + kk;
-        if (j < total) {
-          const long row = ((long)pt[j / PS] * G + g) * PS + j % PS;
-          vreg[i] = *reinterpret_cast<const bf16x8*>(vc + row * Dv + ch * 8);
-        }
+    for (int r = 0; r < 4; ++r) {
+      vreg[r] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
+      const int j = t0 + v_kq * 4 + r;
+      if (v_unit && j < total) {
+        const long row = ((long)pt[j / PS] * G + g) * PS + j % PS;
+        vreg[r] = *reinterpret_cast<const bf16x8*>(vc + row * Dv + v_ch * 8);
       }
     }
   };
@@ -306,15 +305,13 @@ __global__ __launch_bounds__(256) void masked_attn_mfma_kernel(
         *reinterpret_cast<bf16x8*>(k_lds + kk * KS + ch * 8) = kreg[i];
       }
     }
+    if (v_unit) {
+      const int slot = vt_slot(v_kq * 4);
 #pragma unroll
-    for (int i = 0; i < VL; ++i) {
-      const int idx = tid + i * 256;
-      if (idx < KVT * vchunks) {
-        const int kk = idx / vchunks, ch = idx % vchunks;
-        const int slot = vt_slot(kk);
-#pragma unroll
-        for (int e = 0; e < 8; ++e)
-          vt_lds[(ch * 8 + e) * VT_STRIDE + slot] = vreg[i][e];
+      for (int e = 0; e < 8; ++e) {
+        const bf16x4 w4 = {vreg[0][e], vreg[1][e], vreg[2][e], vreg[3][e]};
+        *reinterpret_cast<bf16x4*>(vt_lds + (v_ch * 8 + e) * VT_STRIDE + slot) =
+            w4;
       }
     }
   };
@@ -511,6 +508,17 @@ __global__ __launch_bounds__(256) void masked_attn_decode_kernel(
 
   short* vt = lds + (size_t)wid * Dv * VT_STRIDE;   // this wave's V^T patch
   const int vchunks = Dv / 8;                       // = 2 * nv
+  // this lane's (key quad, chunk) units of a tile's V rows
+  constexpr int VU = (NVB + 3) / 4;
+  int u_kq[VU], u_ch[VU];
+  bool u_ok[VU];
+#pragma unroll
+  for (int it = 0; it < VU; ++it) {
+    const int u = lane + it * WAVE;
+    u_ok[it] = u < 8 * vchunks;
+    u_kq[it] = u / vchunks;
+    u_ch[it] = u % vchunks;
+  }
 
   for (int v = split * 4 + wid; v < n_vt; v += 4 * n_splits) {
     const int kt = v < n_sink ? v : main_first + (v - n_sink);
@@ -531,31 +539,33 @@ __global__ __launch_bounds__(256) void masked_attn_decode_kernel(
           ka[kb][c] = bf16v8{};
       }
     }
-    // V rows, 16 bytes per lane and load
-    bf16x8 vr[NVB];
+    // V: unit = 4 consecutive keys x one 8-value chunk (16 bytes per load)
+    bf16x8 vr[VU][4];
 #pragma unroll
-    for (int i = 0; i < NVB; ++i) {
-      vr[i] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
-      if (i < nv) {
-        const int idx = lane + i * WAVE;
-        const int kk = idx / vchunks, ch = idx % vchunks;
-        const int j = t0 + kk;
-        if (j < total) {
+    for (int it = 0; it < VU; ++it) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        vr[it][r] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
+        const int j = t0 + u_kq[it] * 4 + r;
+        if (u_ok[it] && j < total) {
           const long row = ((long)pt[j / PS] * G + g) * PS + j % PS;
-          vr[i] = *reinterpret_cast<const bf16x8*>(vc + row * Dv + ch * 8);
+          vr[it][r] = *reinterpret_cast<const bf16x8*>(
+              vc + row * Dv + u_ch[it] * 8);
         }
       }
     }
     wave_lds_sync();   // the previous tile's reads of the patch are done
 #pragma unroll
-    for (int i = 0; i < NVB; ++i) {
-      if (i < nv) {
-        const int idx = lane + i * WAVE;
-        const int kk = idx / vchunks, ch = idx % vchunks;
-        const int slot = vt_slot(kk);
+    for (int it = 0; it < VU; ++it) {
+      if (u_ok[it]) {
+        const int slot = vt_slot(u_kq[it] * 4);
 #pragma unroll
-        for (int e = 0; e < 8; ++e)
-          vt[(ch * 8 + e) * VT_STRIDE + slot] = vr[i][e];
+        for (int e = 0; e < 8; ++e) {
+          const bf16x4 w4 = {vr[it][0][e], vr[it][1][e], vr[it][2][e],
+                             vr[it][3][e]};
+          *reinterpret_cast<bf16x4*>(
+              vt + (u_ch[it] * 8 + e) * VT_STRIDE + slot) = w4;
+        }
       }
     }
     wave_lds_sync();

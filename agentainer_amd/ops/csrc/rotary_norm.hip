@@ -14,11 +14,17 @@
 // projection's output); k [T, G, D] goes straight into the pool
 // k_cache[P, G, PS, D] at the token's slot and v [T, G, Dv] is copied into
 // v_cache[P, G, PS, Dv] — rotated keys never travel through HBM twice.
-// slot < 0 skips the append. One wave per (token, head); the head vector
-// sits in a private LDS patch so the pair partner may live in any lane.
+// slot < 0 skips the append. A workgroup serves one token and a slice of
+// its heads (grid.y slices; few slices for long prompts, one head per wave
+// for decode steps): its threads first fill the token's cos/sin table in
+// LDS (the exact, range-reduced cosf/sinf are the expensive part and the
+// heads of a slice share them), then each of the 4 waves takes its heads
+// in turn; a head vector sits in the wave's private LDS patch so the pair
+// partner may live in any lane.
 
 #include <torch/extension.h>
 #include <ATen/hip/HIPContext.h>
+#include <algorithm>
 #include "latent_common.h"
 
 namespace {
@@ -39,58 +45,67 @@ __global__ __launch_bounds__(64 * RN_WAVES) void rotary_norm_append_kernel(
     const float* __restrict__ freqs, float amp, int half,
     const int* __restrict__ positions, const long* __restrict__ slots,
     float eps, const float* __restrict__ q_w, const float* __restrict__ k_w,
-    int norm_first, int n_tok, int H, int G, int D, int Dv, int PS) {
+    int norm_first, int heads_per_wave, int H, int G, int D, int Dv, int PS) {
   extern __shared__ float smem[];
+  float* cs = smem;                            // [2 * half]: cos | sin
   const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
-  const int per_tok = H + 2 * G;
-  const long item = (long)blockIdx.x * RN_WAVES + wave;
-  if (item >= (long)n_tok * per_tok) return;   // whole wave leaves
-  const int t = (int)(item / per_tok), j = (int)(item % per_tok);
-  const long slot = slots[t];
-  if (j >= H + G) {                            // value head: plain copy
-    if (slot < 0) return;
-    const int g = j - H - G;
-    const T* src = v + (long)t * v_ts + (long)g * v_hs;
-    T* dst = v_cache + (((slot / PS) * G + g) * PS + slot % PS) * Dv;
-    for (int i = lane; i < Dv; i += WAVE) dst[i] = src[i];
-    return;
-  }
-  const bool is_q = j < H;
-  if (!is_q && slot < 0) return;
-  float* s = smem + wave * D;
-  const T* src = is_q ? q + (long)t * q_ts + (long)j * q_hs
-                      : k + (long)t * k_ts + (long)(j - H) * k_hs;
-  const float* w = is_q ? q_w : k_w;
-  float ss = 0.f;
-  for (int i = lane; i < D; i += WAVE) {
-    const float u = ldf(src, i);
-    s[i] = u;
-    ss = fmaf(u, u, ss);
-  }
-  if (norm_first) {
-    const float r = 1.0f / sqrtf(wave_sum(ss) / (float)D + eps);
-    for (int i = lane; i < D; i += WAVE)
-      s[i] = s[i] * r * (w != nullptr ? w[i] : 1.0f);
-  }
-  wave_lds_sync();
+  const int t = blockIdx.x;
   const float pos = (float)positions[t];
-  for (int i = lane; i < half; i += WAVE) {
+  for (int i = threadIdx.x; i < half; i += WAVE * RN_WAVES) {
     const float ang = pos * freqs[i];
-    const float c = cosf(ang) * amp, sn = sinf(ang) * amp;
-    const float a = s[i], b = s[i + half];
-    s[i] = a * c - b * sn;
-    s[i + half] = b * c + a * sn;
+    cs[i] = cosf(ang) * amp;
+    cs[half + i] = sinf(ang) * amp;
   }
-  wave_lds_sync();
-  float r = 1.0f;
-  if (!norm_first) {
-    ss = 0.f;
-    for (int i = lane; i < D; i += WAVE) ss = fmaf(s[i], s[i], ss);
-    r = 1.0f / sqrtf(wave_sum(ss) / (float)D + eps);
+  __syncthreads();
+  const long slot = slots[t];
+  float* s = smem + 2 * half + wave * D;
+  const int j0 = (blockIdx.y * RN_WAVES + wave) * heads_per_wave;
+  const int j1 = min(j0 + heads_per_wave, H + 2 * G);
+  for (int j = j0; j < j1; ++j) {              // wave-uniform
+    if (j >= H + G) {                          // value head: plain copy
+      if (slot < 0) continue;
+      const int g = j - H - G;
+      const T* src = v + (long)t * v_ts + (long)g * v_hs;
+      T* dst = v_cache + (((slot / PS) * G + g) * PS + slot % PS) * Dv;
+      for (int i = lane; i < Dv; i += WAVE) dst[i] = src[i];
+      continue;
+    }
+    const bool is_q = j < H;
+    if (!is_q && slot < 0) continue;
+    const T* src = is_q ? q + (long)t * q_ts + (long)j * q_hs
+                        : k + (long)t * k_ts + (long)(j - H) * k_hs;
+    const float* w = is_q ? q_w : k_w;
+    wave_lds_sync();                           // patch free again
+    float ss = 0.f;
+    for (int i = lane; i < D; i += WAVE) {
+      const float u = ldf(src, i);
+      s[i] = u;
+      ss = fmaf(u, u, ss);
+    }
+    if (norm_first) {
+      const float r = 1.0f / sqrtf(wave_sum(ss) / (float)D + eps);
+      for (int i = lane; i < D; i += WAVE)
+        s[i] = s[i] * r * (w != nullptr ? w[i] : 1.0f);
+    }
+    wave_lds_sync();
+    for (int i = lane; i < half; i += WAVE) {
+      const float c = cs[i], sn = cs[half + i];
+      const float a = s[i], b = s[i + half];
+      s[i] = a * c - b * sn;
+      s[i + half] = b * c + a * sn;
+    }
+    wave_lds_sync();
+    float r = 1.0f;
+    if (!norm_first) {
+      ss = 0.f;
+      for (int i = lane; i < D; i += WAVE) ss = fmaf(s[i], s[i], ss);
+      r = 1.0f / sqrtf(wave_sum(ss) / (float)D + eps);
+    }
+    T* dst = is_q ? q + (long)t * q_ts + (long)j * q_hs
+                  : k_cache +
+                        (((slot / PS) * G + (j - H)) * PS + slot % PS) * D;
+    for (int i = lane; i < D; i += WAVE) stf(dst, i, s[i] * r);
   }
-  T* dst = is_q ? q + (long)t * q_ts + (long)j * q_hs
-                : k_cache + (((slot / PS) * G + (j - H)) * PS + slot % PS) * D;
-  for (int i = lane; i < D; i += WAVE) stf(dst, i, s[i] * r);
 }
 
 }  // namespace
@@ -141,20 +156,24 @@ void rotary_norm_append(torch::Tensor q, torch::Tensor k, torch::Tensor v,
     kw = k_w->data_ptr<float>();
   }
   if (T_ == 0) return;
-  const long items = (long)T_ * (H + 2 * G);
-  const size_t smem = (size_t)RN_WAVES * D * sizeof(float);
+  const size_t smem = ((size_t)RN_WAVES * D + 2 * half) * sizeof(float);
   TORCH_CHECK(smem <= 64 * 1024, "head size too large");
+  // long prompts: several heads per wave share one cos/sin table; short
+  // steps: one head per wave so the launch still fills the chip
+  const int per_tok = H + 2 * G;
+  const int hpw = T_ >= 1024 ? std::min(4, (per_tok + RN_WAVES - 1) / RN_WAVES)
+                             : 1;
+  const int slices = (per_tok + RN_WAVES * hpw - 1) / (RN_WAVES * hpw);
   auto stream = at::hip::getCurrentHIPStream();
   LATENT_DISPATCH_T(q, {
     hipLaunchKernelGGL(
         rotary_norm_append_kernel<T>,
-        dim3((unsigned)((items + RN_WAVES - 1) / RN_WAVES)),
-        dim3(64 * RN_WAVES), smem, stream, (T*)q.data_ptr(), (long)q.stride(0),
+        dim3((unsigned)T_, (unsigned)slices), dim3(64 * RN_WAVES), smem, stream, (T*)q.data_ptr(), (long)q.stride(0),
         (long)q.stride(1), (const T*)k.data_ptr(), (long)k.stride(0),
         (long)k.stride(1), (const T*)v.data_ptr(), (long)v.stride(0),
         (long)v.stride(1), (T*)k_cache.data_ptr(), (T*)v_cache.data_ptr(),
         freqs.data_ptr<float>(), (float)amp, half, positions.data_ptr<int>(),
         slot_mapping.data_ptr<long>(), (float)eps, qw, kw,
-        norm_first ? 1 : 0, T_, H, G, D, Dv, (int)k_cache.size(2));
+        norm_first ? 1 : 0, hpw, H, G, D, Dv, (int)k_cache.size(2));
   });
 }

@@ -89,23 +89,44 @@ __global__ __launch_bounds__(256) void scalar_rmsnorm_kernel(
   }
 }
 
-template <typename T, int VEC>
+// MAXC > 0: the row (F <= 256 * VEC * MAXC values) is held in registers
+// between the two passes, so z is read from memory once; MAXC == 0 re-reads.
+template <typename T, int VEC, int MAXC>
 __global__ __launch_bounds__(256) void poly_norm_kernel(
     T* __restrict__ out, const T* __restrict__ z, long z_rs,
     const float* __restrict__ coef, float eps, int F) {
   __shared__ float red[4];
   const long row = blockIdx.x;
   const T* zr = z + row * z_rs;
+  constexpr int NC = MAXC > 0 ? MAXC : 1;
+  float keep[NC][VEC];
   float s2 = 0.f, s4 = 0.f, s6 = 0.f;
-  for (int i = threadIdx.x * VEC; i < F; i += 256 * VEC) {
-    float v[VEC];
-    ldv<T, VEC>(zr, i, v);
+  if constexpr (MAXC > 0) {
 #pragma unroll
-    for (int j = 0; j < VEC; ++j) {
-      const float q = v[j] * v[j];
-      s2 += q;
-      s4 = fmaf(q, q, s4);
-      s6 = fmaf(q * v[j], q * v[j], s6);
+    for (int c = 0; c < MAXC; ++c) {
+      const int i = (c * 256 + threadIdx.x) * VEC;
+      if (i < F) {
+        ldv<T, VEC>(zr, i, keep[c]);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+          const float q = keep[c][j] * keep[c][j];
+          s2 += q;
+          s4 = fmaf(q, q, s4);
+          s6 = fmaf(q * keep[c][j], q * keep[c][j], s6);
+        }
+      }
+    }
+  } else {
+    for (int i = threadIdx.x * VEC; i < F; i += 256 * VEC) {
+      float v[VEC];
+      ldv<T, VEC>(zr, i, v);
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        const float q = v[j] * v[j];
+        s2 += q;
+        s4 = fmaf(q, q, s4);
+        s6 = fmaf(q * v[j], q * v[j], s6);
+      }
     }
   }
   const float n = (float)F;
@@ -114,15 +135,31 @@ __global__ __launch_bounds__(256) void poly_norm_kernel(
   const float r3 = coef[2] / sqrtf(block_sum_256(s6, red) / n + eps);
   const float e = coef[3];
   T* orow = out + row * F;
-  for (int i = threadIdx.x * VEC; i < F; i += 256 * VEC) {
-    float v[VEC];
-    ldv<T, VEC>(zr, i, v);
+  if constexpr (MAXC > 0) {
 #pragma unroll
-    for (int j = 0; j < VEC; ++j) {
-      const float q = v[j] * v[j];
-      v[j] = fmaf(v[j], r1, fmaf(q, r2, fmaf(q * v[j], r3, e)));
+    for (int c = 0; c < MAXC; ++c) {
+      const int i = (c * 256 + threadIdx.x) * VEC;
+      if (i < F) {
+        float v[VEC];
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+          const float x = keep[c][j], q = x * x;
+          v[j] = fmaf(x, r1, fmaf(q, r2, fmaf(q * x, r3, e)));
+        }
+        stv<T, VEC>(orow, i, v);
+      }
     }
-    stv<T, VEC>(orow, i, v);
+  } else {
+    for (int i = threadIdx.x * VEC; i < F; i += 256 * VEC) {
+      float v[VEC];
+      ldv<T, VEC>(zr, i, v);
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        const float q = v[j] * v[j];
+        v[j] = fmaf(v[j], r1, fmaf(q, r2, fmaf(q * v[j], r3, e)));
+      }
+      stv<T, VEC>(orow, i, v);
+    }
   }
 }
 
@@ -202,17 +239,20 @@ void poly_norm(torch::Tensor out, torch::Tensor z, torch::Tensor coef,
   const bool vec = F % 4 == 0 && z.stride(0) % 4 == 0 && aligned16(z) &&
                    aligned16(out);
   auto stream = at::hip::getCurrentHIPStream();
+#define LAUNCH_POLY(VEC_, MAXC_)                                              \
+  hipLaunchKernelGGL((poly_norm_kernel<T, VEC_, MAXC_>), dim3(T_), dim3(256), \
+                     0, stream, (T*)out.data_ptr(), (const T*)z.data_ptr(),   \
+                     (long)z.stride(0), coef.data_ptr<float>(), (float)eps, F)
   LATENT_DISPATCH_T(z, {
-    if (vec) {
-      hipLaunchKernelGGL((poly_norm_kernel<T, 4>), dim3(T_), dim3(256), 0,
-                         stream, (T*)out.data_ptr(), (const T*)z.data_ptr(),
-                         (long)z.stride(0), coef.data_ptr<float>(), (float)eps,
-                         F);
+    if (vec && F <= 256 * 4 * 4) {
+      LAUNCH_POLY(4, 4);
+    } else if (vec && F <= 256 * 4 * 16) {
+      LAUNCH_POLY(4, 16);
+    } else if (vec) {
+      LAUNCH_POLY(4, 0);
     } else {
-      hipLaunchKernelGGL((poly_norm_kernel<T, 1>), dim3(T_), dim3(256), 0,
-                         stream, (T*)out.data_ptr(), (const T*)z.data_ptr(),
-                         (long)z.stride(0), coef.data_ptr<float>(), (float)eps,
-                         F);
+      LAUNCH_POLY(1, 0);
     }
   });
+#undef LAUNCH_POLY
 }
