@@ -27,7 +27,9 @@ Serving design (what runs on the MI355X):
 
   * q, k, v (and the head-gate logits) come out of ONE GEMM; one fused
     kernel (ops.rotary_norm_append) rotates / normalizes q in place and k
-    on its way into the paged pool and copies v there. The engine's
+    on its way into the paged pool and copies v there. The cos/sin rows of
+    a step's positions (ops.rotary_table, fp32 angles) are computed once
+    per step and rotary setting and shared by all layers that have it. The engine's
     KVCacheManager owns the pools through HeadKVLayout — per layer
     K [pages, G, page, dim] and V [pages, G, page, vdim].
   * ops.masked_attention serves prompt portions and single decoded tokens
@@ -232,9 +234,24 @@ class MaskedAttention(torch.nn.Module):
             self.key_bias.copy_(get("pb").float())
         self.w_o.copy_(get("o"))
 
-    def forward(self, h: torch.Tensor, k_cache: torch.Tensor,
-                v_cache: torch.Tensor, md: AttnMetadata) -> torch.Tensor:
+    def rotary_key(self):
+        """Layers with equal keys share one cos/sin table per step."""
         mc = self.mc
+        sc = mc.rot_scaling
+        return (mc.rot_dims, mc.rot_base,
+                tuple(sorted(sc.items())) if sc else None)
+
+    def forward(self, h: torch.Tensor, k_cache: torch.Tensor,
+                v_cache: torch.Tensor, md: AttnMetadata,
+                tables: Optional[dict] = None) -> torch.Tensor:
+        mc = self.mc
+        key = self.rotary_key()
+        cos_sin = tables.get(key) if tables is not None else None
+        if cos_sin is None:
+            cos_sin = ops.rotary_table(md.positions, self.rot_freqs,
+                                       self.rot_amp)
+            if tables is not None:
+                tables[key] = cos_sin
         T, H, G = h.size(0), mc.heads, mc.kv_heads
         proj = ops.linear(h, self.w_in, bias=self.b_in)
         k0, v0 = self.q_sz, self.q_sz + self.k_sz
@@ -243,10 +260,9 @@ class MaskedAttention(torch.nn.Module):
         q = proj[:, :k0].view(T, H, mc.dim)
         k = proj[:, k0:v0].view(T, G, mc.dim)
         v = proj[:, v0:g0].view(T, G, mc.vdim)
-        ops.rotary_norm_append(q, k, v, k_cache, v_cache, self.rot_freqs,
-                               self.rot_amp, md.positions, md.slot_mapping,
-                               self.eps, self.q_norm, self.k_norm,
-                               mc.norm_first)
+        ops.rotary_norm_append(q, k, v, k_cache, v_cache, cos_sin,
+                               md.slot_mapping, self.eps, self.q_norm,
+                               self.k_norm, mc.norm_first)
         out = torch.empty(T, H, mc.vdim, dtype=h.dtype, device=h.device)
         ops.masked_attention(
             out, q, k_cache, v_cache, md.page_table, md.seq_lens,
@@ -391,9 +407,11 @@ class VolalornForCausalLM(torch.nn.Module):
             ops.scalar_postnorm_residual(x, y, gain, eps, nxt)
             return nxt
 
+        tables: dict = {}      # rotary setting -> this step's cos/sin rows
         for i, layer in enumerate(self.layers):
             k_cache, v_cache = kv_caches[i]
-            h = add_normed(layer.mix(h, k_cache, v_cache, md), layer.norm1)
+            h = add_normed(layer.mix(h, k_cache, v_cache, md, tables),
+                           layer.norm1)
             if layer.mlp is not None:
                 h = add_normed(layer.mlp(h), layer.norm2)
             if self.residual_trace is not None:

@@ -607,18 +607,25 @@ def poly_norm(out, z, coef, eps: float):
     return out
 
 
-def rotary_norm_append(q, k, v, k_cache, v_cache, freqs, amp: float,
-                       positions, slot_mapping, eps: float, q_w=None,
-                       k_w=None, norm_first: bool = False):
+def rotary_table(positions, freqs, amp: float):
+    """fp32 [T, 2*half]: cos | sin of positions[t] * freqs[i], times amp."""
+    mod = _dispatch_masked("rotary_table", positions)
+    if mod:
+        return mod.rotary_table(positions, freqs, float(amp))
+    return reference.rotary_table(positions, freqs, amp)
+
+
+def rotary_norm_append(q, k, v, k_cache, v_cache, cos_sin, slot_mapping,
+                       eps: float, q_w=None, k_w=None,
+                       norm_first: bool = False):
     mod = _dispatch_masked("rotary_norm_append", q)
     if mod:
-        mod.rotary_norm_append(q, k, v, k_cache, v_cache, freqs, float(amp),
-                               positions, slot_mapping, float(eps), q_w, k_w,
+        mod.rotary_norm_append(q, k, v, k_cache, v_cache, cos_sin,
+                               slot_mapping, float(eps), q_w, k_w,
                                bool(norm_first))
     else:
-        reference.rotary_norm_append(q, k, v, k_cache, v_cache, freqs, amp,
-                                     positions, slot_mapping, eps, q_w, k_w,
-                                     norm_first)
+        reference.rotary_norm_append(q, k, v, k_cache, v_cache, cos_sin,
+                                     slot_mapping, eps, q_w, k_w, norm_first)
 
 
 # AGENTAINER_MASKED_SIMPLE=1 forces the one-wave-per-row kernel (A/B and

@@ -8,10 +8,11 @@ void scalar_rmsnorm(torch::Tensor out, torch::Tensor x, torch::Tensor gain,
                     double eps);
 void poly_norm(torch::Tensor out, torch::Tensor z, torch::Tensor coef,
                double eps);
+torch::Tensor rotary_table(torch::Tensor positions, torch::Tensor freqs,
+                           double amp);
 void rotary_norm_append(torch::Tensor q, torch::Tensor k, torch::Tensor v,
                         torch::Tensor k_cache, torch::Tensor v_cache,
-                        torch::Tensor freqs, double amp,
-                        torch::Tensor positions, torch::Tensor slot_mapping,
+                        torch::Tensor cos_sin, torch::Tensor slot_mapping,
                         double eps, c10::optional<torch::Tensor> q_w,
                         c10::optional<torch::Tensor> k_w, bool norm_first);
 void masked_attention(torch::Tensor out, torch::Tensor q, torch::Tensor k_cache,
@@ -31,6 +32,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         "x += gain * y / rms(y); h = x in the compute dtype");
   m.def("scalar_rmsnorm", &scalar_rmsnorm, "gain * x / rms(x)");
   m.def("poly_norm", &poly_norm, "a U(z) + b U(z^2) + c U(z^3) + e");
+  m.def("rotary_table", &rotary_table,
+        "cos | sin of position * frequency for one step's tokens");
   m.def("rotary_norm_append", &rotary_norm_append,
         "rotary + q/k rms norm; append K/V to the paged pools");
   m.def("masked_attention", &masked_attention,

@@ -1,26 +1,27 @@
-// Query/key preparation fused with the paged K/V append (gfx950).
+// Rotary tables and query/key preparation fused with the paged K/V append
+// (gfx950).
 //
-// For every new token and head, in fp32:
+//   rotary_table         cs[t] = (cos(a) * amp | sin(a) * amp), a = position
+//                        * freq[i] (fp32 product, exact range-reduced
+//                        cosf/sinf), once per engine step and rotary setting:
+//                        every layer and head with that setting reads it.
+//   rotary_norm_append   for every new token and head, in fp32:
 //
-//   norm_first : u <- u / sqrt(mean(u^2) + eps) * w ;  u <- rotate(u)
-//   otherwise  : u <- rotate(u) ;  u <- u / sqrt(mean(u^2) + eps)
+//     norm_first : u <- u / sqrt(mean(u^2) + eps) * w ;  u <- rotate(u)
+//     otherwise  : u <- rotate(u) ;  u <- u / sqrt(mean(u^2) + eps)
 //
-// rotate() turns the first 2*half coordinates of the head: coordinate i is
-// paired with i + half, angle = position * freq[i] (fp32 product, exact
-// cosf/sinf), and cos/sin are scaled by `amp` (1 unless the frequencies
-// are YaRN-stretched). Coordinates from 2*half on pass through.
+// rotate() turns the first 2*half coordinates of the head, coordinate i
+// paired with i + half; coordinates from 2*half on pass through. `amp` is 1
+// unless the frequencies are YaRN-stretched.
 //
 // q [T, H, D] is rewritten in place (a strided view of the fused
 // projection's output); k [T, G, D] goes straight into the pool
 // k_cache[P, G, PS, D] at the token's slot and v [T, G, Dv] is copied into
 // v_cache[P, G, PS, Dv] — rotated keys never travel through HBM twice.
-// slot < 0 skips the append. A workgroup serves one token and a slice of
-// its heads (grid.y slices; few slices for long prompts, one head per wave
-// for decode steps): its threads first fill the token's cos/sin table in
-// LDS (the exact, range-reduced cosf/sinf are the expensive part and the
-// heads of a slice share them), then each of the 4 waves takes its heads
-// in turn; a head vector sits in the wave's private LDS patch so the pair
-// partner may live in any lane.
+// slot < 0 skips the append. One wave per (token, head): a lane owns whole
+// rotation pairs (i, i + half) plus a strided share of the pass-through
+// coordinates, so a head lives in registers from its load to its store and
+// only the sums of squares cross lanes.
 
 #include <torch/extension.h>
 #include <ATen/hip/HIPContext.h>
@@ -30,11 +31,19 @@
 namespace {
 
 constexpr int RN_WAVES = 4;
+constexpr int RN_PAIRS = 2;   // rotation pairs per lane: rotary dims <= 256
+constexpr int RN_PASS = 4;    // pass-through values per lane: <= 256
 
-__device__ __forceinline__ void wave_lds_sync() {
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-  __builtin_amdgcn_wave_barrier();
-  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+__global__ __launch_bounds__(256) void rotary_table_kernel(
+    float* __restrict__ cs, const int* __restrict__ positions,
+    const float* __restrict__ freqs, float amp, int half, long n) {
+  const long idx = (long)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= n) return;
+  const long t = idx / half;
+  const int i = (int)(idx % half);
+  const float ang = (float)positions[t] * freqs[i];
+  cs[t * 2 * half + i] = cosf(ang) * amp;
+  cs[t * 2 * half + half + i] = sinf(ang) * amp;
 }
 
 template <typename T>
@@ -42,26 +51,20 @@ __global__ __launch_bounds__(64 * RN_WAVES) void rotary_norm_append_kernel(
     T* __restrict__ q, long q_ts, long q_hs, const T* __restrict__ k,
     long k_ts, long k_hs, const T* __restrict__ v, long v_ts, long v_hs,
     T* __restrict__ k_cache, T* __restrict__ v_cache,
-    const float* __restrict__ freqs, float amp, int half,
-    const int* __restrict__ positions, const long* __restrict__ slots,
-    float eps, const float* __restrict__ q_w, const float* __restrict__ k_w,
-    int norm_first, int heads_per_wave, int H, int G, int D, int Dv, int PS) {
-  extern __shared__ float smem[];
-  float* cs = smem;                            // [2 * half]: cos | sin
+    const float* __restrict__ cos_sin, int half,
+    const long* __restrict__ slots, float eps, const float* __restrict__ q_w,
+    const float* __restrict__ k_w, int norm_first, int n_tok, int H, int G,
+    int D, int Dv, int PS) {
   const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
-  const int t = blockIdx.x;
-  const float pos = (float)positions[t];
-  for (int i = threadIdx.x; i < half; i += WAVE * RN_WAVES) {
-    const float ang = pos * freqs[i];
-    cs[i] = cosf(ang) * amp;
-    cs[half + i] = sinf(ang) * amp;
-  }
-  __syncthreads();
+  const int per_tok = H + 2 * G;
+  const unsigned item = blockIdx.x * RN_WAVES + wave;
+  if (item >= (unsigned)n_tok * per_tok) return;   // whole wave leaves
+  const int t = (int)(item / (unsigned)per_tok);
+  const float* cs = cos_sin + (long)t * 2 * half;
   const long slot = slots[t];
-  float* s = smem + 2 * half + wave * D;
-  const int j0 = (blockIdx.y * RN_WAVES + wave) * heads_per_wave;
-  const int j1 = min(j0 + heads_per_wave, H + 2 * G);
-  for (int j = j0; j < j1; ++j) {              // wave-uniform
+  const int rot = 2 * half;
+  const int j0 = (int)(item % (unsigned)per_tok);
+  for (int j = j0; j == j0; ++j) {             // one item; `continue` leaves
     if (j >= H + G) {                          // value head: plain copy
       if (slot < 0) continue;
       const int g = j - H - G;
@@ -75,45 +78,103 @@ __global__ __launch_bounds__(64 * RN_WAVES) void rotary_norm_append_kernel(
     const T* src = is_q ? q + (long)t * q_ts + (long)j * q_hs
                         : k + (long)t * k_ts + (long)(j - H) * k_hs;
     const float* w = is_q ? q_w : k_w;
-    wave_lds_sync();                           // patch free again
+    // every load of the head is issued before the first use: head values,
+    // the token's cos/sin and (norm_first) the norm weights
+    float a[RN_PAIRS], b[RN_PAIRS], c[RN_PASS];
+    float cc[RN_PAIRS], sn[RN_PAIRS];
+    float wa[RN_PAIRS], wb[RN_PAIRS], wc[RN_PASS];
+    const bool use_w = norm_first && w != nullptr;
+#pragma unroll
+    for (int n = 0; n < RN_PAIRS; ++n) {
+      const int i = lane + n * WAVE;
+      const bool ok = i < half;
+      a[n] = ok ? ldf(src, i) : 0.f;
+      b[n] = ok ? ldf(src, i + half) : 0.f;
+      cc[n] = ok ? cs[i] : 1.f;
+      sn[n] = ok ? cs[half + i] : 0.f;
+      wa[n] = (ok && use_w) ? w[i] : 1.f;
+      wb[n] = (ok && use_w) ? w[i + half] : 1.f;
+    }
+#pragma unroll
+    for (int n = 0; n < RN_PASS; ++n) {
+      const int i = rot + lane + n * WAVE;
+      c[n] = i < D ? ldf(src, i) : 0.f;
+      wc[n] = (i < D && use_w) ? w[i] : 1.f;
+    }
     float ss = 0.f;
-    for (int i = lane; i < D; i += WAVE) {
-      const float u = ldf(src, i);
-      s[i] = u;
-      ss = fmaf(u, u, ss);
-    }
     if (norm_first) {
+#pragma unroll
+      for (int n = 0; n < RN_PAIRS; ++n)
+        ss = fmaf(a[n], a[n], fmaf(b[n], b[n], ss));
+#pragma unroll
+      for (int n = 0; n < RN_PASS; ++n) ss = fmaf(c[n], c[n], ss);
       const float r = 1.0f / sqrtf(wave_sum(ss) / (float)D + eps);
-      for (int i = lane; i < D; i += WAVE)
-        s[i] = s[i] * r * (w != nullptr ? w[i] : 1.0f);
+#pragma unroll
+      for (int n = 0; n < RN_PAIRS; ++n) {
+        a[n] *= r * wa[n];
+        b[n] *= r * wb[n];
+      }
+#pragma unroll
+      for (int n = 0; n < RN_PASS; ++n) c[n] *= r * wc[n];
     }
-    wave_lds_sync();
-    for (int i = lane; i < half; i += WAVE) {
-      const float c = cs[i], sn = cs[half + i];
-      const float a = s[i], b = s[i + half];
-      s[i] = a * c - b * sn;
-      s[i + half] = b * c + a * sn;
+    ss = 0.f;
+#pragma unroll
+    for (int n = 0; n < RN_PAIRS; ++n) {
+      const float x = a[n], y = b[n];
+      a[n] = x * cc[n] - y * sn[n];
+      b[n] = y * cc[n] + x * sn[n];
+      ss = fmaf(a[n], a[n], fmaf(b[n], b[n], ss));
     }
-    wave_lds_sync();
     float r = 1.0f;
     if (!norm_first) {
-      ss = 0.f;
-      for (int i = lane; i < D; i += WAVE) ss = fmaf(s[i], s[i], ss);
+#pragma unroll
+      for (int n = 0; n < RN_PASS; ++n) ss = fmaf(c[n], c[n], ss);
       r = 1.0f / sqrtf(wave_sum(ss) / (float)D + eps);
     }
     T* dst = is_q ? q + (long)t * q_ts + (long)j * q_hs
                   : k_cache +
                         (((slot / PS) * G + (j - H)) * PS + slot % PS) * D;
-    for (int i = lane; i < D; i += WAVE) stf(dst, i, s[i] * r);
+#pragma unroll
+    for (int n = 0; n < RN_PAIRS; ++n) {
+      const int i = lane + n * WAVE;
+      if (i < half) {
+        stf(dst, i, a[n] * r);
+        stf(dst, i + half, b[n] * r);
+      }
+    }
+#pragma unroll
+    for (int n = 0; n < RN_PASS; ++n) {
+      const int i = rot + lane + n * WAVE;
+      if (i < D) stf(dst, i, c[n] * r);
+    }
   }
 }
 
 }  // namespace
 
+torch::Tensor rotary_table(torch::Tensor positions, torch::Tensor freqs,
+                           double amp) {
+  TORCH_CHECK(positions.scalar_type() == at::kInt && positions.is_contiguous() &&
+              positions.is_cuda());
+  TORCH_CHECK(freqs.scalar_type() == at::kFloat && freqs.is_contiguous() &&
+              freqs.device() == positions.device());
+  const long T_ = positions.numel();
+  const int half = freqs.numel();
+  auto cs = torch::empty({T_, 2L * half},
+                         torch::TensorOptions().dtype(torch::kFloat).device(
+                             positions.device()));
+  const long n = T_ * half;
+  if (n == 0) return cs;
+  hipLaunchKernelGGL(rotary_table_kernel, dim3((unsigned)((n + 255) / 256)),
+                     dim3(256), 0, at::hip::getCurrentHIPStream(),
+                     cs.data_ptr<float>(), positions.data_ptr<int>(),
+                     freqs.data_ptr<float>(), (float)amp, half, n);
+  return cs;
+}
+
 void rotary_norm_append(torch::Tensor q, torch::Tensor k, torch::Tensor v,
                         torch::Tensor k_cache, torch::Tensor v_cache,
-                        torch::Tensor freqs, double amp,
-                        torch::Tensor positions, torch::Tensor slot_mapping,
+                        torch::Tensor cos_sin, torch::Tensor slot_mapping,
                         double eps, c10::optional<torch::Tensor> q_w,
                         c10::optional<torch::Tensor> k_w, bool norm_first) {
   TORCH_CHECK(q.dim() == 3 && k.dim() == 3 && v.dim() == 3 &&
@@ -135,12 +196,12 @@ void rotary_norm_append(torch::Tensor q, torch::Tensor k, torch::Tensor v,
               k_cache.scalar_type() == q.scalar_type() &&
               v_cache.scalar_type() == q.scalar_type(),
               "q, k, v and the pools share one element type");
-  TORCH_CHECK(freqs.scalar_type() == at::kFloat && freqs.is_contiguous() &&
-              freqs.is_cuda());
-  const int half = freqs.numel();
+  TORCH_CHECK(cos_sin.scalar_type() == at::kFloat && cos_sin.is_contiguous() &&
+              cos_sin.dim() == 2 && cos_sin.size(0) == T_ &&
+              cos_sin.size(1) % 2 == 0 && cos_sin.is_cuda(),
+              "cos_sin must be contiguous fp32 [T, 2 * half]");
+  const int half = cos_sin.size(1) / 2;
   TORCH_CHECK(2 * half <= D, "rotary dims exceed the head size");
-  TORCH_CHECK(positions.scalar_type() == at::kInt && positions.numel() == T_ &&
-              positions.is_contiguous());
   TORCH_CHECK(slot_mapping.scalar_type() == at::kLong &&
               slot_mapping.numel() == T_ && slot_mapping.is_contiguous());
   const float* qw = nullptr;
@@ -156,24 +217,21 @@ void rotary_norm_append(torch::Tensor q, torch::Tensor k, torch::Tensor v,
     kw = k_w->data_ptr<float>();
   }
   if (T_ == 0) return;
-  const size_t smem = ((size_t)RN_WAVES * D + 2 * half) * sizeof(float);
-  TORCH_CHECK(smem <= 64 * 1024, "head size too large");
-  // long prompts: several heads per wave share one cos/sin table; short
-  // steps: one head per wave so the launch still fills the chip
-  const int per_tok = H + 2 * G;
-  const int hpw = T_ >= 1024 ? std::min(4, (per_tok + RN_WAVES - 1) / RN_WAVES)
-                             : 1;
-  const int slices = (per_tok + RN_WAVES * hpw - 1) / (RN_WAVES * hpw);
+  TORCH_CHECK(half <= WAVE * RN_PAIRS && D - 2 * half <= WAVE * RN_PASS,
+              "head size too large");
+  const long items = (long)T_ * (H + 2 * G);
+  TORCH_CHECK(items < (1L << 31), "too many (token, head) items");
   auto stream = at::hip::getCurrentHIPStream();
   LATENT_DISPATCH_T(q, {
     hipLaunchKernelGGL(
         rotary_norm_append_kernel<T>,
-        dim3((unsigned)T_, (unsigned)slices), dim3(64 * RN_WAVES), smem, stream, (T*)q.data_ptr(), (long)q.stride(0),
+        dim3((unsigned)((items + RN_WAVES - 1) / RN_WAVES)),
+        dim3(64 * RN_WAVES), 0, stream, (T*)q.data_ptr(), (long)q.stride(0),
         (long)q.stride(1), (const T*)k.data_ptr(), (long)k.stride(0),
         (long)k.stride(1), (const T*)v.data_ptr(), (long)v.stride(0),
         (long)v.stride(1), (T*)k_cache.data_ptr(), (T*)v_cache.data_ptr(),
-        freqs.data_ptr<float>(), (float)amp, half, positions.data_ptr<int>(),
-        slot_mapping.data_ptr<long>(), (float)eps, qw, kw,
-        norm_first ? 1 : 0, hpw, H, G, D, Dv, (int)k_cache.size(2));
+        cos_sin.data_ptr<float>(), half, slot_mapping.data_ptr<long>(),
+        (float)eps, qw, kw, norm_first ? 1 : 0, T_, H, G, D, Dv,
+        (int)k_cache.size(2));
   });
 }

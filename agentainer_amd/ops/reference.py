@@ -385,22 +385,28 @@ def rotary_frequencies(dims: int, base: float, scaling=None, device=None):
     return f.to(device), float(amp)
 
 
-def _rotate_half(u: torch.Tensor, positions: torch.Tensor,
-                 freqs: torch.Tensor, amp: float) -> torch.Tensor:
-    """u fp32 [T, heads, D]; the first 2*len(freqs) coordinates of every
-    head rotate, coordinate i paired with i + len(freqs)."""
-    half = freqs.numel()
+def rotary_table(positions: torch.Tensor, freqs: torch.Tensor,
+                 amp: float) -> torch.Tensor:
+    """fp32 [T, 2*half] = cos(a) * amp | sin(a) * amp with a = position *
+    freq in fp32: one row per token of the step, shared by every layer and
+    head with this rotary setting."""
     ang = positions.to(torch.float32).unsqueeze(1) * freqs.unsqueeze(0)
-    c = (torch.cos(ang) * amp).unsqueeze(1)
-    s = (torch.sin(ang) * amp).unsqueeze(1)
+    return torch.cat([torch.cos(ang) * amp, torch.sin(ang) * amp], dim=1)
+
+
+def _rotate_half(u: torch.Tensor, cos_sin: torch.Tensor) -> torch.Tensor:
+    """u fp32 [T, heads, D]; the first 2*half coordinates of every head
+    rotate, coordinate i paired with i + half; cos_sin [T, 2*half]."""
+    half = cos_sin.size(1) // 2
+    c = cos_sin[:, :half].unsqueeze(1)
+    s = cos_sin[:, half:].unsqueeze(1)
     a, b = u[..., :half], u[..., half:2 * half]
     return torch.cat([a * c - b * s, b * c + a * s, u[..., 2 * half:]], -1)
 
 
 def rotary_norm_append(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
                        k_cache: torch.Tensor, v_cache: torch.Tensor,
-                       freqs: torch.Tensor, amp: float,
-                       positions: torch.Tensor, slot_mapping: torch.Tensor,
+                       cos_sin: torch.Tensor, slot_mapping: torch.Tensor,
                        eps: float, q_w=None, k_w=None,
                        norm_first: bool = False) -> None:
     """Prepare one step's queries and keys and append K/V to the pools.
@@ -408,7 +414,7 @@ def rotary_norm_append(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
     q [T, H, D] (rewritten in place), k [T, G, D], v [T, G, Dv]; pools
     k_cache [P, G, PS, D], v_cache [P, G, PS, Dv] (per page and kv head, PS
     consecutive token rows); slot = page*PS + offset (slot < 0 skips the
-    append). Per head, in fp32:
+    append); cos_sin = rotary_table(...) of the step. Per head, in fp32:
       norm_first: u <- rms_norm(u) * w, then rotate   (w = q_w / k_w [D])
       otherwise : u <- rotate(u), then unit rms (no weight)."""
     def prep(u, w):
@@ -417,8 +423,8 @@ def rotary_norm_append(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
             u = _unit(u, eps)
             if w is not None:
                 u = u * w.float()
-            return _rotate_half(u, positions, freqs, amp)
-        return _unit(_rotate_half(u, positions, freqs, amp), eps)
+            return _rotate_half(u, cos_sin)
+        return _unit(_rotate_half(u, cos_sin), eps)
 
     q.copy_(prep(q, q_w).to(q.dtype))
     kk = prep(k, k_w).to(k_cache.dtype)

@@ -89,13 +89,15 @@ def test_rotary_norm_append(dtype, norm_first, H, G, D, Dv, rot):
     pr = proj.clone()
     kc_r = torch.full((P, G, PS, D), 7.0, dtype=dtype)
     vc_r = torch.full((P, G, PS, Dv), 7.0, dtype=dtype)
-    ref.rotary_norm_append(*views(pr), kc_r, vc_r, freqs, amp, pos, slots,
-                           1e-5, qw, kw, norm_first)
+    cs_r = ref.rotary_table(pos, freqs, amp)
+    ref.rotary_norm_append(*views(pr), kc_r, vc_r, cs_r, slots, 1e-5, qw, kw,
+                           norm_first)
     pd = proj.cuda()
     kc_d = torch.full((P, G, PS, D), 7.0, dtype=dtype, device="cuda")
     vc_d = torch.full((P, G, PS, Dv), 7.0, dtype=dtype, device="cuda")
-    ops.rotary_norm_append(*views(pd), kc_d, vc_d, freqs.cuda(), amp,
-                           pos.cuda(), slots.cuda(), 1e-5,
+    cs_d = ops.rotary_table(pos.cuda(), freqs.cuda(), amp)
+    torch.testing.assert_close(cs_d.cpu(), cs_r, rtol=5e-4, atol=5e-4)
+    ops.rotary_norm_append(*views(pd), kc_d, vc_d, cs_d, slots.cuda(), 1e-5,
                            qw.cuda() if norm_first else None,
                            kw.cuda() if norm_first else None, norm_first)
     # fp32 angles of a few thousand radians: cos/sin agree to ~1e-4

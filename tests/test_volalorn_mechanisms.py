@@ -125,8 +125,8 @@ def test_rotary_norm_append(device, norm_first, H, G, D, Dv, rot):
     kc = torch.zeros(P, G, PS, D, device=device)
     vc = torch.zeros(P, G, PS, Dv, device=device)
     qd = q.clone().to(device)
-    ops.rotary_norm_append(qd, k.to(device), v.to(device), kc, vc,
-                           freqs.to(device), amp, pos.to(device),
+    cs = ops.rotary_table(pos.to(device), freqs.to(device), amp)
+    ops.rotary_norm_append(qd, k.to(device), v.to(device), kc, vc, cs,
                            slots.to(device), 1e-4,
                            qw.to(device) if norm_first else None,
                            kw.to(device) if norm_first else None, norm_first)
