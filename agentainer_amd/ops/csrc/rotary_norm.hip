@@ -150,6 +150,133 @@ __global__ __launch_bounds__(64 * RN_WAVES) void rotary_norm_append_kernel(
   }
 }
 
+
+// bf16 heads of exactly 64 * EPL coordinates (EPL = 1, 2, 4; rotary half a
+// multiple of EPL): lane l owns coordinates [l*EPL, (l+1)*EPL), moved with
+// ONE load and ONE store per head, and takes its rotation partner from lane
+// l +- half/EPL by a shuffle. The kernel is bound by vector-memory
+// instructions per wave, and this form issues 4-5 of them instead of 11.
+template <int EPL>
+struct VecOf;
+template <>
+struct VecOf<1> { typedef short S; typedef float F; };
+template <>
+struct VecOf<2> {
+  typedef short S __attribute__((ext_vector_type(2)));
+  typedef float F __attribute__((ext_vector_type(2)));
+};
+template <>
+struct VecOf<4> {
+  typedef short S __attribute__((ext_vector_type(4)));
+  typedef float F __attribute__((ext_vector_type(4)));
+};
+
+template <int EPL>
+__device__ __forceinline__ void ld_bf(const short* p, float* v) {
+  typename VecOf<EPL>::S t = *reinterpret_cast<const typename VecOf<EPL>::S*>(p);
+  if constexpr (EPL == 1) {
+    v[0] = bits2f(t);
+  } else {
+#pragma unroll
+    for (int e = 0; e < EPL; ++e) v[e] = bits2f(t[e]);
+  }
+}
+template <int EPL>
+__device__ __forceinline__ void st_bf(short* p, const float* v) {
+  typename VecOf<EPL>::S t;
+  if constexpr (EPL == 1) {
+    t = f2bits(v[0]);
+  } else {
+#pragma unroll
+    for (int e = 0; e < EPL; ++e) t[e] = f2bits(v[e]);
+  }
+  *reinterpret_cast<typename VecOf<EPL>::S*>(p) = t;
+}
+template <int EPL>
+__device__ __forceinline__ void ld_f(const float* p, float* v) {
+  typename VecOf<EPL>::F t = *reinterpret_cast<const typename VecOf<EPL>::F*>(p);
+  if constexpr (EPL == 1) {
+    v[0] = t;
+  } else {
+#pragma unroll
+    for (int e = 0; e < EPL; ++e) v[e] = t[e];
+  }
+}
+
+template <int EPL>
+__global__ __launch_bounds__(64 * RN_WAVES) void rotary_norm_append_vec_kernel(
+    short* __restrict__ q, long q_ts, long q_hs, const short* __restrict__ k,
+    long k_ts, long k_hs, const short* __restrict__ v, long v_ts, long v_hs,
+    short* __restrict__ k_cache, short* __restrict__ v_cache,
+    const float* __restrict__ cos_sin, int half,
+    const long* __restrict__ slots, float eps, const float* __restrict__ q_w,
+    const float* __restrict__ k_w, int norm_first, int n_tok, int H, int G,
+    int Dv, int PS) {
+  constexpr int D = WAVE * EPL;
+  const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+  const int per_tok = H + 2 * G;
+  const unsigned item = blockIdx.x * RN_WAVES + wave;
+  if (item >= (unsigned)n_tok * per_tok) return;   // whole wave leaves
+  const int t = (int)(item / (unsigned)per_tok);
+  const int j = (int)(item % (unsigned)per_tok);
+  const long slot = slots[t];
+  if (j >= H + G) {                            // value head: plain copy
+    if (slot < 0) return;
+    const int g = j - H - G;
+    const short* src = v + (long)t * v_ts + (long)g * v_hs;
+    short* dst = v_cache + (((slot / PS) * G + g) * PS + slot % PS) * Dv;
+    for (int i = lane; i < Dv; i += WAVE) dst[i] = src[i];
+    return;
+  }
+  const bool is_q = j < H;
+  if (!is_q && slot < 0) return;
+  const short* src = is_q ? q + (long)t * q_ts + (long)j * q_hs
+                          : k + (long)t * k_ts + (long)(j - H) * k_hs;
+  const float* w = is_q ? q_w : k_w;
+  const int e0 = lane * EPL;
+  const int rot = 2 * half;
+  const bool low = e0 < half, turns = e0 < rot;
+  const float* cs = cos_sin + (long)t * rot;
+  float x[EPL], cc[EPL], sn[EPL], wv[EPL];
+  ld_bf<EPL>(src + e0, x);
+#pragma unroll
+  for (int e = 0; e < EPL; ++e) { cc[e] = 1.f; sn[e] = 0.f; wv[e] = 1.f; }
+  if (turns) {
+    const int i0 = low ? e0 : e0 - half;
+    ld_f<EPL>(cs + i0, cc);
+    ld_f<EPL>(cs + half + i0, sn);
+  }
+  if (norm_first && w != nullptr) ld_f<EPL>(w + e0, wv);
+  if (norm_first) {
+    float ss = 0.f;
+#pragma unroll
+    for (int e = 0; e < EPL; ++e) ss = fmaf(x[e], x[e], ss);
+    const float r = 1.0f / sqrtf(wave_sum(ss) / (float)D + eps);
+#pragma unroll
+    for (int e = 0; e < EPL; ++e) x[e] *= r * wv[e];
+  }
+  // partner coordinate e +- half lives half/EPL lanes away
+  const int hop = half / EPL;
+  const int partner = low ? lane + hop : lane - hop;
+  float ss = 0.f;
+#pragma unroll
+  for (int e = 0; e < EPL; ++e) {
+    const float y = __shfl(x[e], turns ? partner : lane, WAVE);
+    const float rx = low ? x[e] * cc[e] - y * sn[e] : x[e] * cc[e] + y * sn[e];
+    x[e] = turns ? rx : x[e];
+    ss = fmaf(x[e], x[e], ss);
+  }
+  if (!norm_first) {
+    const float r = 1.0f / sqrtf(wave_sum(ss) / (float)D + eps);
+#pragma unroll
+    for (int e = 0; e < EPL; ++e) x[e] *= r;
+  }
+  short* dst = is_q ? q + (long)t * q_ts + (long)j * q_hs
+                    : k_cache +
+                          (((slot / PS) * G + (j - H)) * PS + slot % PS) * D;
+  st_bf<EPL>(dst + e0, x);
+}
+
 }  // namespace
 
 torch::Tensor rotary_table(torch::Tensor positions, torch::Tensor freqs,
@@ -222,11 +349,43 @@ void rotary_norm_append(torch::Tensor q, torch::Tensor k, torch::Tensor v,
   const long items = (long)T_ * (H + 2 * G);
   TORCH_CHECK(items < (1L << 31), "too many (token, head) items");
   auto stream = at::hip::getCurrentHIPStream();
+  const dim3 grid((unsigned)((items + RN_WAVES - 1) / RN_WAVES));
+  const int epl = D / WAVE;
+  auto al = [&](const torch::Tensor& x, long bytes) {
+    return reinterpret_cast<uintptr_t>(x.data_ptr()) % bytes == 0;
+  };
+  if (q.scalar_type() == at::kBFloat16 && D % WAVE == 0 &&
+      (epl == 1 || epl == 2 || epl == 4) && half % epl == 0 &&
+      q.stride(0) % epl == 0 && q.stride(1) % epl == 0 &&
+      k.stride(0) % epl == 0 && k.stride(1) % epl == 0 && al(q, 2 * epl) &&
+      al(k, 2 * epl) && al(k_cache, 2 * epl) && al(cos_sin, 16) &&
+      (qw == nullptr || reinterpret_cast<uintptr_t>(qw) % 16 == 0) &&
+      (kw == nullptr || reinterpret_cast<uintptr_t>(kw) % 16 == 0)) {
+#define LAUNCH_VEC(EPL_)                                                      \
+  hipLaunchKernelGGL(                                                         \
+      rotary_norm_append_vec_kernel<EPL_>, grid, dim3(64 * RN_WAVES), 0,      \
+      stream, (short*)q.data_ptr(), (long)q.stride(0), (long)q.stride(1),     \
+      (const short*)k.data_ptr(), (long)k.stride(0), (long)k.stride(1),       \
+      (const short*)v.data_ptr(), (long)v.stride(0), (long)v.stride(1),       \
+      (short*)k_cache.data_ptr(), (short*)v_cache.data_ptr(),                 \
+      cos_sin.data_ptr<float>(), half, slot_mapping.data_ptr<long>(),         \
+      (float)eps, qw, kw, norm_first ? 1 : 0, T_, H, G, Dv,                   \
+      (int)k_cache.size(2))
+    if (epl == 1) {
+      LAUNCH_VEC(1);
+    } else if (epl == 2) {
+      LAUNCH_VEC(2);
+    } else {
+      LAUNCH_VEC(4);
+    }
+#undef LAUNCH_VEC
+    return;
+  }
   LATENT_DISPATCH_T(q, {
     hipLaunchKernelGGL(
         rotary_norm_append_kernel<T>,
-        dim3((unsigned)((items + RN_WAVES - 1) / RN_WAVES)),
-        dim3(64 * RN_WAVES), 0, stream, (T*)q.data_ptr(), (long)q.stride(0),
+        grid, dim3(64 * RN_WAVES), 0, stream, (T*)q.data_ptr(),
+        (long)q.stride(0),
         (long)q.stride(1), (const T*)k.data_ptr(), (long)k.stride(0),
         (long)k.stride(1), (const T*)v.data_ptr(), (long)v.stride(0),
         (long)v.stride(1), (T*)k_cache.data_ptr(), (T*)v_cache.data_ptr(),

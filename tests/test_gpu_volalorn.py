@@ -66,12 +66,16 @@ def test_poly_norm(dtype, F_):
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("norm_first", [False, True])
 @pytest.mark.parametrize("H,G,D,Dv,rot", [(4, 2, 64, 32, 32), (6, 3, 96, 40, 96),
-                                          (3, 1, 20, 12, 8), (8, 8, 128, 128, 64)])
+                                          (3, 1, 20, 12, 8), (8, 8, 128, 128, 64),
+                                          (5, 1, 128, 24, 128), (2, 1, 256, 64, 64),
+                                          (2, 2, 64, 8, 2), (1, 1, 128, 16, 0)])
 def test_rotary_norm_append(dtype, norm_first, H, G, D, Dv, rot):
     g = torch.Generator().manual_seed(D + H)
     T, PS, P = 29, 4, 12
     n = H * D + G * D + G * Dv
-    proj = torch.randn(T, n + 3, generator=g).to(dtype)
+    # odd row stride for odd head sizes; 16-byte rows where the one-load
+    # form of the kernel applies (64 / 128 / 256 coordinates per head)
+    proj = torch.randn(T, n + (3 if D % 64 else 8), generator=g).to(dtype)
     pos = torch.randint(0, 3000, (T,), generator=g, dtype=torch.int32)
     slots = torch.randperm(P * PS, generator=g)[:T]
     slots[5] = -1
