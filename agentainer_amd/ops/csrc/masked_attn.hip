@@ -60,6 +60,36 @@ __device__ __forceinline__ float sigmoidf_(float x) {
   return 1.0f / (1.0f + expf(-x));
 }
 
+// bf16 tile kernels: hardware exp2 / rcp forms (relative error ~1e-6, far
+// below the bf16 rounding of the weights they produce)
+__device__ __forceinline__ float fast_exp(float x) { return __expf(x); }
+__device__ __forceinline__ float fast_sigmoid(float x) {
+  return __fdividef(1.0f, 1.0f + __expf(-x));
+}
+__device__ __forceinline__ float fast_tanh(float x) {
+  return 2.0f * fast_sigmoid(2.0f * x) - 1.0f;
+}
+
+// token position -> (page index in the sequence's table, row in the page);
+// page sizes that are powers of two (ps_shift >= 0) avoid the division
+__device__ __forceinline__ void page_of(int j, int PS, int ps_shift, int& pg,
+                                        int& off) {
+  if (ps_shift >= 0) {
+    pg = j >> ps_shift;
+    off = j & (PS - 1);
+  } else {
+    pg = j / PS;
+    off = j % PS;
+  }
+}
+
+__device__ __forceinline__ bf16v8 pack_bf16(const float* v) {
+  bf16v8 r;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) r[e] = (__bf16)v[e];
+  return r;
+}
+
 // ------------------------------------------------------------------
 // masked_attn_rowwave: one wave per (query token, head)
 // ------------------------------------------------------------------
@@ -190,7 +220,7 @@ __global__ __launch_bounds__(256) void masked_attn_mfma_kernel(
     const int* __restrict__ q_lens, float scale, int kind, int size, int keep,
     int sigmoid_w, float softcap, const float* __restrict__ key_bias,
     const short* __restrict__ gate, long g_ts, int H, int G, int nd, int nv,
-    int PS, int max_pages) {
+    int PS, int max_pages, int ps_shift) {
   extern __shared__ __attribute__((aligned(16))) short lds[];
   constexpr int KL = NDB / 2;              // 16-byte K loads per thread
   const int D = nd * 32, Dv = nv * 16;
@@ -220,6 +250,7 @@ __global__ __launch_bounds__(256) void masked_attn_mfma_kernel(
   }
   const int ctx = total - qlen;
   const int* pt = page_table + (long)b * max_pages;
+  const float inv_cap = softcap > 0.f ? 1.0f / softcap : 0.f;
 
   // ---- key tiles of this block: kept prefix + main range of its columns
   const int c_last = min(c0 + COLS_PER_BLOCK, ncols) - 1;
@@ -281,7 +312,9 @@ __global__ __launch_bounds__(256) void masked_attn_mfma_kernel(
         const int kk = idx / kchunks, ch = idx % kchunks;
         const int j = t0 + kk;
         if (j < total) {
-          const long row = ((long)pt[j / PS] * G + g) * PS + j % PS;
+          int pg, off;
+          page_of(j, PS, ps_shift, pg, off);
+          const long row = ((long)pt[pg] * G + g) * PS + off;
           kreg[i] = *reinterpret_cast<const bf16x8*>(kc + row * D + ch * 8);
         }
       }
@@ -291,7 +324,9 @@ __global__ __launch_bounds__(256) void masked_attn_mfma_kernel(
       vreg[r] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
       const int j = t0 + v_kq * 4 + r;
       if (v_unit && j < total) {
-        const long row = ((long)pt[j / PS] * G + g) * PS + j % PS;
+        int pg, off;
+        page_of(j, PS, ps_shift, pg, off);
+        const long row = ((long)pt[pg] * G + g) * PS + off;
         vreg[r] = *reinterpret_cast<const bf16x8*>(vc + row * Dv + v_ch * 8);
       }
     }
@@ -353,14 +388,14 @@ __global__ __launch_bounds__(256) void masked_attn_mfma_kernel(
         const int j = t0 + (e >> 2) * 16 + lg * 4 + (e & 3);
         vis[e] = j <= qpos && (j >= lo || j < keep);
         float s = sv[e] * scale;
-        if (softcap > 0.f) s = softcap * tanhf(s / softcap);
+        if (softcap > 0.f) s = softcap * fast_tanh(s * inv_cap);
         sv[e] = s;
       }
       float pv[8];
       if (sigmoid_w) {
 #pragma unroll
         for (int e = 0; e < 8; ++e)
-          pv[e] = vis[e] ? sigmoidf_(sv[e] + bias) : 0.f;
+          pv[e] = vis[e] ? fast_sigmoid(sv[e] + bias) : 0.f;
       } else {
         float tm = -FLT_MAX;
 #pragma unroll
@@ -368,11 +403,11 @@ __global__ __launch_bounds__(256) void masked_attn_mfma_kernel(
         tm = fmaxf(tm, __shfl_xor(tm, 16, WAVE));
         tm = fmaxf(tm, __shfl_xor(tm, 32, WAVE));
         const float mn = fmaxf(m, tm);
-        const float alpha = (m == -FLT_MAX) ? 0.f : expf(m - mn);
+        const float alpha = (m == -FLT_MAX) ? 0.f : fast_exp(m - mn);
         float ts = 0.f;
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
-          pv[e] = vis[e] ? expf(sv[e] - mn) : 0.f;
+          pv[e] = vis[e] ? fast_exp(sv[e] - mn) : 0.f;
           ts += pv[e];
         }
         ts += __shfl_xor(ts, 16, WAVE);
@@ -384,11 +419,7 @@ __global__ __launch_bounds__(256) void masked_attn_mfma_kernel(
           if (i < nv) o[i] *= alpha;
       }
       // P^T as the second MFMA's B operand, straight from registers
-      bf16x8 pb;
-#pragma unroll
-      for (int e = 0; e < 8; ++e) pb[e] = f2bits(pv[e]);
-      bf16v8 pf;
-      __builtin_memcpy(&pf, &pb, 16);
+      const bf16v8 pf = pack_bf16(pv);
       // ---- O^T += V^T P^T
 #pragma unroll
       for (int i = 0; i < NVB; ++i) {
@@ -450,7 +481,7 @@ __global__ __launch_bounds__(256) void masked_attn_decode_kernel(
     const int* __restrict__ seq_lens, float scale, int kind, int size, int keep,
     int sigmoid_w, float softcap, const float* __restrict__ key_bias,
     const short* __restrict__ gate, long g_ts, int H, int G, int nd, int nv,
-    int PS, int max_pages, float* __restrict__ part_o,
+    int PS, int max_pages, int ps_shift, float* __restrict__ part_o,
     float* __restrict__ part_ml, int n_splits) {
   extern __shared__ __attribute__((aligned(16))) short lds[];
   const int D = nd * 32, Dv = nv * 16;
@@ -480,6 +511,7 @@ __global__ __launch_bounds__(256) void masked_attn_decode_kernel(
   const int qpos = total - 1;
   const int lo = mask_lo(qpos, kind, size);
   const int* pt = page_table + (long)b * max_pages;
+  const float inv_cap = softcap > 0.f ? 1.0f / softcap : 0.f;
   const int kt_end = qpos / KVT + 1;
   const int main_first = lo / KVT;
   const int n_sink = min((keep + KVT - 1) / KVT, main_first);
@@ -506,7 +538,10 @@ __global__ __launch_bounds__(256) void masked_attn_decode_kernel(
   for (int i = 0; i < NVB; ++i) o[i] = f32x4{0.f, 0.f, 0.f, 0.f};
   float m = -FLT_MAX, l = 0.f;
 
-  short* vt = lds + (size_t)wid * Dv * VT_STRIDE;   // this wave's V^T patch
+  // this wave's V^T patch: [Dv][32 keys] with no padding (4 workgroups of
+  // 4 waves fit a CU's LDS); the 16-byte unit inside a row is XOR-ed with
+  // bits of the row so the A-fragment reads of 16 rows spread over all banks
+  short* vt = lds + (size_t)wid * Dv * KVT;
   const int vchunks = Dv / 8;                       // = 2 * nv
   // this lane's (key quad, chunk) units of a tile's V rows
   constexpr int VU = (NVB + 3) / 4;
@@ -529,7 +564,9 @@ __global__ __launch_bounds__(256) void masked_attn_decode_kernel(
     for (int kb = 0; kb < 2; ++kb) {
       const int j = t0 + kb * 16 + l16;
       const bool ok = j < total;
-      const long row = ok ? ((long)pt[j / PS] * G + g) * PS + j % PS : 0;
+      int pg, off;
+      page_of(ok ? j : 0, PS, ps_shift, pg, off);
+      const long row = ((long)pt[pg] * G + g) * PS + off;
       const short* kr = kc + row * D + lg * 8;
 #pragma unroll
       for (int c = 0; c < NDB; ++c) {
@@ -543,14 +580,30 @@ __global__ __launch_bounds__(256) void masked_attn_decode_kernel(
     bf16x8 vr[VU][4];
 #pragma unroll
     for (int it = 0; it < VU; ++it) {
+      const int jq = t0 + u_kq[it] * 4;
+      if ((PS & 3) == 0) {       // the four keys of a unit share a page
+        int pg, off;
+        page_of(jq < total ? jq : 0, PS, ps_shift, pg, off);
+        const short* vrow =
+            vc + (((long)pt[pg] * G + g) * PS + off) * Dv + u_ch[it] * 8;
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        vr[it][r] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
-        const int j = t0 + u_kq[it] * 4 + r;
-        if (u_ok[it] && j < total) {
-          const long row = ((long)pt[j / PS] * G + g) * PS + j % PS;
-          vr[it][r] = *reinterpret_cast<const bf16x8*>(
-              vc + row * Dv + u_ch[it] * 8);
+        for (int r = 0; r < 4; ++r) {
+          vr[it][r] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
+          if (u_ok[it] && jq + r < total)
+            vr[it][r] = *reinterpret_cast<const bf16x8*>(vrow + r * Dv);
+        }
+      } else {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          vr[it][r] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
+          const int j = jq + r;
+          if (u_ok[it] && j < total) {
+            int pg, off;
+            page_of(j, PS, ps_shift, pg, off);
+            const long row = ((long)pt[pg] * G + g) * PS + off;
+            vr[it][r] = *reinterpret_cast<const bf16x8*>(
+                vc + row * Dv + u_ch[it] * 8);
+          }
         }
       }
     }
@@ -563,8 +616,10 @@ __global__ __launch_bounds__(256) void masked_attn_decode_kernel(
         for (int e = 0; e < 8; ++e) {
           const bf16x4 w4 = {vr[it][0][e], vr[it][1][e], vr[it][2][e],
                              vr[it][3][e]};
+          const int row = u_ch[it] * 8 + e;
           *reinterpret_cast<bf16x4*>(
-              vt + (u_ch[it] * 8 + e) * VT_STRIDE + slot) = w4;
+              vt + row * KVT + (((slot >> 3) ^ ((row >> 2) & 3)) << 3) +
+              (slot & 7)) = w4;
         }
       }
     }
@@ -589,13 +644,13 @@ __global__ __launch_bounds__(256) void masked_attn_decode_kernel(
       const int j = t0 + (e >> 2) * 16 + lg * 4 + (e & 3);
       vis[e] = j <= cq && (j >= lo || j < keep);
       float s = sv[e] * scale;
-      if (softcap > 0.f) s = softcap * tanhf(s / softcap);
+      if (softcap > 0.f) s = softcap * fast_tanh(s * inv_cap);
       sv[e] = s;
     }
     if (sigmoid_w) {
 #pragma unroll
       for (int e = 0; e < 8; ++e)
-        pv[e] = vis[e] ? sigmoidf_(sv[e] + bias) : 0.f;
+        pv[e] = vis[e] ? fast_sigmoid(sv[e] + bias) : 0.f;
     } else {
       float tm = -FLT_MAX;
 #pragma unroll
@@ -603,11 +658,11 @@ __global__ __launch_bounds__(256) void masked_attn_decode_kernel(
       tm = fmaxf(tm, __shfl_xor(tm, 16, WAVE));
       tm = fmaxf(tm, __shfl_xor(tm, 32, WAVE));
       const float mn = fmaxf(m, tm);
-      const float alpha = (m == -FLT_MAX) ? 0.f : expf(m - mn);
+      const float alpha = (m == -FLT_MAX) ? 0.f : fast_exp(m - mn);
       float ts = 0.f;
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
-        pv[e] = vis[e] ? expf(sv[e] - mn) : 0.f;
+        pv[e] = vis[e] ? fast_exp(sv[e] - mn) : 0.f;
         ts += pv[e];
       }
       ts += __shfl_xor(ts, 16, WAVE);
@@ -618,16 +673,13 @@ __global__ __launch_bounds__(256) void masked_attn_decode_kernel(
       for (int i = 0; i < NVB; ++i)
         if (i < nv) o[i] *= alpha;
     }
-    bf16x8 pb;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) pb[e] = f2bits(pv[e]);
-    bf16v8 pf;
-    __builtin_memcpy(&pf, &pb, 16);
+    const bf16v8 pf = pack_bf16(pv);
 #pragma unroll
     for (int i = 0; i < NVB; ++i) {
       if (i < nv) {
+        const int row = i * 16 + l16;
         const bf16v8 af = *reinterpret_cast<const bf16v8*>(
-            vt + (i * 16 + l16) * VT_STRIDE + lg * 8);
+            vt + row * KVT + ((lg ^ ((row >> 2) & 3)) << 3));
         o[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af, pf, o[i], 0, 0, 0);
       }
     }
@@ -788,6 +840,9 @@ void masked_attention(torch::Tensor out, torch::Tensor q, torch::Tensor k_cache,
       aligned16(k_cache.data_ptr()) && aligned16(v_cache.data_ptr());
   if (mfma_ok) {
     const int nd = D / 32, nv = Dv / 16;
+    int ps_shift = -1;
+    if ((PS & (PS - 1)) == 0)
+      for (ps_shift = 0; (1 << ps_shift) < PS; ++ps_shift) {}
     const short* gp =
         head_gate.has_value() ? (const short*)head_gate->data_ptr() : nullptr;
     if (!query_starts.has_value() && R <= 16) {
@@ -809,7 +864,7 @@ void masked_attention(torch::Tensor out, torch::Tensor q, torch::Tensor k_cache,
         pmlp = pml.data_ptr<float>();
       }
       const dim3 dgrid((unsigned)n_splits, B, G);
-      const size_t dlds = (size_t)4 * Dv * VT_STRIDE * 2 + 512;
+      const size_t dlds = (size_t)4 * Dv * KVT * 2 + 512;
 #define LAUNCH_DECODE(NDB_, NVB_)                                             \
   hipLaunchKernelGGL((masked_attn_decode_kernel<NDB_, NVB_>), dgrid,          \
                      dim3(256), dlds, stream, (short*)out.data_ptr(),         \
@@ -820,7 +875,8 @@ void masked_attention(torch::Tensor out, torch::Tensor q, torch::Tensor k_cache,
                      page_table.data_ptr<int>(), seq_lens.data_ptr<int>(),    \
                      (float)scale, (int)mask_kind, (int)mask_size, keep,      \
                      sigmoid_weights ? 1 : 0, (float)softcap, kb, gp, g_ts, H, \
-                     G, nd, nv, PS, max_pages, pop, pmlp, (int)n_splits)
+                     G, nd, nv, PS, max_pages, ps_shift, pop, pmlp,     \
+                     (int)n_splits)
       if (nd <= 4 && nv <= 4) {
         LAUNCH_DECODE(4, 4);
       } else if (nd <= 4 && nv <= 8) {
@@ -850,7 +906,7 @@ void masked_attention(torch::Tensor out, torch::Tensor q, torch::Tensor k_cache,
                      page_table.data_ptr<int>(), seq_lens.data_ptr<int>(), qs, \
                      ql, (float)scale, (int)mask_kind, (int)mask_size, keep,  \
                      sigmoid_weights ? 1 : 0, (float)softcap, kb, gp, g_ts, H, \
-                     G, nd, nv, PS, max_pages)
+                     G, nd, nv, PS, max_pages, ps_shift)
     if (nd <= 4 && nv <= 4) {
       LAUNCH_MFMA(4, 4);
     } else if (nd <= 4 && nv <= 8) {
