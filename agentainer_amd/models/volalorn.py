@@ -432,7 +432,7 @@ def _tiny(name: str) -> VolalornConfig:
         heads=4, kv_heads=2, dim=32, vdim=32, scale=32 ** -0.5,
         mask_kind=ops.MASK_CHUNK, mask_size=32, rot_dims=16,
         rot_base=10000.0, rot_scaling={"factor": 4.0, "original": 256,
-                                       "fast": 32.0, "slow": 1.0},
+                                       "fast": 16.0, "slow": 2.0},
         softcap=30.0, sigmoid_weights=True, key_bias=True, head_gate=True)
     soft = MaskedAttentionConfig(
         heads=4, kv_heads=1, dim=32, vdim=16, scale=32 ** -0.5,
@@ -442,7 +442,7 @@ def _tiny(name: str) -> VolalornConfig:
               VolalornLayerConfig("attention_2", soft,
                                   PolyFeedForwardConfig(256))]
     return VolalornConfig(name=name, vocab_size=512, hidden_size=128,
-                          layers=layers, norm_eps=1e-6, logit_scale=0.5)
+                          layers=layers, norm_eps=1e-5, logit_scale=0.75)
 
 
 VOLALORN_CONFIGS: Dict[str, VolalornConfig] = {

@@ -138,7 +138,7 @@ def _arch_points():
 def _volalorn_points():
     """Volalorn size points beside Llama stacks of equal width, head counts
     and ff: layers alternate the sigmoid/chunk mixer (YaRN rotary on half
-    the head) and the softmax/window mixer (4 kept first tokens). Masks are
+    the head) and the softmax/window mixer (8 kept first tokens). Masks are
     sized so that a decode step at the benchmark's context reads about as
     many keys as the Llama stack does."""
     from agentainer_amd import ops
@@ -152,19 +152,19 @@ def _volalorn_points():
         sig = MaskedAttentionConfig(
             heads=heads, kv_heads=kv, dim=128, vdim=128, scale=128 ** -0.5,
             mask_kind=ops.MASK_CHUNK, mask_size=chunk, rot_dims=64,
-            rot_base=500000.0, rot_scaling={"factor": 8.0, "original": 8192,
-                                            "fast": 32.0, "slow": 1.0},
+            rot_base=500000.0, rot_scaling={"factor": 4.0, "original": 8192,
+                                            "fast": 16.0, "slow": 2.0},
             softcap=30.0, sigmoid_weights=True, key_bias=True, head_gate=True)
         soft = MaskedAttentionConfig(
             heads=heads, kv_heads=kv, dim=128, vdim=128, scale=128 ** -0.5,
-            mask_kind=ops.MASK_WINDOW, mask_size=window, keep_first=4,
+            mask_kind=ops.MASK_WINDOW, mask_size=window, keep_first=8,
             rot_dims=128, rot_base=500000.0, qkv_bias=True, norm_first=True)
         layers = [VolalornLayerConfig(
             "attention" if i % 2 == 0 else "attention_2",
             sig if i % 2 == 0 else soft, PolyFeedForwardConfig(ff))
             for i in range(n)]
         return VolalornConfig(name=name, vocab_size=32000, hidden_size=width,
-                              layers=layers, norm_eps=1e-6, logit_scale=0.5)
+                              layers=layers, norm_eps=1e-5, logit_scale=0.75)
 
     return {
         "s": ("w2048-ff8192", vol("volalorn-s", 2048, 16, 4, 2048, 1024,
