@@ -149,15 +149,18 @@ MASKS = [
 
 @pytest.mark.parametrize("simple", [False, True])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
-@pytest.mark.parametrize("H,G,D,Dv", [(4, 2, 64, 32), (6, 2, 64, 48),
-                                      (8, 1, 32, 16), (2, 2, 256, 256),
-                                      (3, 1, 20, 12), (5, 5, 96, 80)])
+@pytest.mark.parametrize("H,G,D,Dv,PS", [
+    (4, 2, 64, 32, 16), (6, 2, 64, 48, 16), (8, 1, 32, 16, 16),
+    (2, 2, 256, 256, 16), (3, 1, 20, 12, 16), (5, 5, 96, 80, 16),
+    # more heads per kv head than one wave's 16 columns; page sizes that
+    # are not powers of two (with and without whole four-key units)
+    (40, 2, 32, 32, 16), (4, 1, 64, 64, 12), (2, 1, 32, 16, 6)])
 @pytest.mark.parametrize("mask", MASKS)
-def test_masked_attention_prompt_and_decode(simple, dtype, H, G, D, Dv, mask):
+def test_masked_attention_prompt_and_decode(simple, dtype, H, G, D, Dv, PS,
+                                            mask):
     if simple and dtype == torch.float32:
         pytest.skip("fp32 always takes the row kernel")
     kind, size, keep, sig, cap, use_gate = mask
-    PS = 16
     lens = [1, 200, 77, 131, 64]
     qlens = [1, 150, 2, 131, 1]
     (q, kc, vc, pt, sl, qs, ql, gate, bias) = _attn_case(
